@@ -1,2 +1,2 @@
 """Architectures known to the registry."""
-from . import qwen2  # noqa: F401
+from . import qwen2, volonex  # noqa: F401

@@ -101,11 +101,27 @@ def stop_token_ids(model_dir: str | None, config: "ModelConfig") -> list[int]:
 
 
 def architecture_name(data: dict) -> str:
-    """architectures[0], the name the registry is keyed by."""
+    """The name the registry is keyed by: architectures[0], or the string under 'architecture'."""
     archs = data.get("architectures")
     if isinstance(archs, list) and archs and isinstance(archs[0], str):
         return archs[0]
-    raise ConfigError("config key 'architectures' must be a non-empty list of names")
+    one = data.get("architecture")
+    if isinstance(one, str) and one:
+        return one
+    raise ConfigError("config key 'architectures' must be a non-empty list of names "
+                      "(or 'architecture' a name)")
+
+
+def read_object(data: dict, key: str, default: Any = REQUIRED) -> dict | None:
+    """data[key] as a nested object; a missing or null key gives the default or an error."""
+    value = data.get(key)
+    if value is None:
+        if default is REQUIRED:
+            raise ConfigError(f"config key '{key}' is required")
+        return default
+    if not isinstance(value, dict):
+        raise ConfigError(f"config key '{key}': expected an object, got {value!r}")
+    return value
 
 
 @dataclasses.dataclass

@@ -6,9 +6,13 @@
 // prompt steps and one-token steps give identical bits. It is the 32-bit path's attention and
 // the reference beside the MFMA kernels.
 //
-// For the query at absolute position p: first = window > 0 ? max(0, p+1-window) : 0,
+// For the query at absolute position p: first = window > 0 ? max(0, p+1-window) : 0, and with
+// chunk > 0 no earlier than the start of p's chunk, p - p % chunk (chunks are counted from position 0);
 // s_j = (q . k_j) * scale for j in [first, p], out = sum_j softmax(s)_j v_j,
 // kv head = h / (H / KVH)   (reference: kernels/attention.cu:155-316, :664-773, :60).
+// sinks (one number a head, or null): the softmax's denominator also holds exp(sink_h), which has no
+// key and no value; it joins last, after the pages. gate (one number a row and head, or null): the
+// head's output is multiplied by sigmoid(gate) before it is stored.
 //
 // Three launches keep that order and give the same bits: one wavefront per (query, head) that walks
 // the pages itself (or, in a step of many queries, per four neighbouring queries, which share what
@@ -23,6 +27,13 @@
 #include "hector_kernels.h"
 
 #define AP_MAX_PER_LANE 8
+
+// the first key the query at position p sees
+__device__ __forceinline__ int ap_first(int p, int window, int chunk) {
+  int first = window > 0 ? max(0, p + 1 - window) : 0;
+  if (chunk > 0) first = max(first, p - p % chunk);
+  return first;
+}
 
 // NPL: head elements a lane holds (head_dim / 64 rounded up to 1, 2, 4 or 8)
 template <int NPL>
@@ -136,6 +147,28 @@ __device__ __forceinline__ void ap_join(ApState<NPL>& total, const ApState<NPL>&
   total.m = m_new;
 }
 
+// What a (row, head) is finished with: the sink joins the softmax, the gate scales the output.
+struct ApExtras {
+  const void* sinks;     // [H] or null
+  int sinks_dtype;
+  const void* gate;      // gate[row * gate_stride + h] in the activation dtype, or null
+  int64_t gate_stride;
+};
+template <typename T, int NPL>
+__device__ __forceinline__ float ap_finish(ApState<NPL>& total, const ApExtras& ex, int64_t row, int h) {
+  if (ex.sinks != nullptr) {
+    ApState<NPL> sk;
+    sk.m = load_param(ex.sinks, h, ex.sinks_dtype);
+    sk.l = 1.f;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) sk.acc[i] = 0.f;
+    ap_join(total, sk);
+  }
+  if (ex.gate == nullptr) return 1.f;
+  const float g = to_float(((const T*)ex.gate)[row * ex.gate_stride + h]);
+  return 1.f / (1.f + expf(-g));
+}
+
 // grid (rows, ceil(H / 4), pages): pages == 1: the wavefront walks all pages of its query and stores
 // the result; pages > 1: it takes the page (first >> 6) + blockIdx.z alone and stores (m, l, sums)
 // into ws [row][head][pages][hd + 2], if the query has such a page.
@@ -145,7 +178,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
     const T* __restrict__ vpool, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ page_table, int max_blocks, int num_pages, int H, int KVH, int hd,
-    int window, float scale) {
+    int window, int chunk, float scale, ApExtras ex) {
   const int lane = threadIdx.x & (HE_WAVE - 1);
   const int h = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int64_t row = blockIdx.x;
@@ -165,7 +198,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
   const int p = positions[row];
   const int slot = seq_slot[seq];
   const int kvh = h / (H / KVH);
-  const int first = window > 0 ? max(0, p + 1 - window) : 0;
+  const int first = ap_first(p, window, chunk);
   const int32_t* pt = page_table + (int64_t)slot * max_blocks;
   const int c_first = first >> HE_PAGE_SHIFT, c_last = p >> HE_PAGE_SHIFT;
   if (split && c_first + (int)blockIdx.z > c_last) return;
@@ -201,11 +234,12 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
                min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
     ap_join(total, st);
   }
+  const float gf = ap_finish<T, NPL>(total, ex, row, h);
   const float inv = total.l > 0.f ? 1.f / total.l : 0.f;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     const int d = lane + i * HE_WAVE;
-    if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
+    if (i < npl && d < hd) o[d] = from_float<T>(ex.gate ? total.acc[i] * inv * gf : total.acc[i] * inv);
   }
 }
 
@@ -220,7 +254,7 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kpool, const T* __restrict__ vpool,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
-    int num_pages, int rows, int H, int KVH, int hd, int window, float scale) {
+    int num_pages, int rows, int H, int KVH, int hd, int window, int chunk, float scale, ApExtras ex) {
   const int lane = threadIdx.x & (HE_WAVE - 1);
   const int h = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (h >= H) return;
@@ -231,13 +265,14 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
   const int seq0 = row_seq[row0], p0 = positions[row0];
   bool together = n_rows == AP_ROWS && seq0 >= 0;
   for (int r = 1; r < n_rows; ++r) together = together && row_seq[row0 + r] == seq0 && positions[row0 + r] == p0 + r;
-  auto store = [&](int64_t row, const ApState<NPL>& total) {
+  auto store = [&](int64_t row, ApState<NPL>& total) {
     T* o = out + (row * H + h) * (int64_t)hd;
+    const float gf = row_seq[row] >= 0 ? ap_finish<T, NPL>(total, ex, row, h) : 1.f;
     const float inv = total.l > 0.f ? 1.f / total.l : 0.f;
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
       const int d = lane + i * HE_WAVE;
-      if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
+      if (i < npl && d < hd) o[d] = from_float<T>(ex.gate ? total.acc[i] * inv * gf : total.acc[i] * inv);
     }
   };
   auto load_q = [&](float (&qv)[NPL], int64_t row) {
@@ -259,7 +294,7 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
       const int seq = row_seq[row];
       if (seq >= 0) {
         const int p = positions[row];
-        const int first = window > 0 ? max(0, p + 1 - window) : 0;
+        const int first = ap_first(p, window, chunk);
         const int32_t* pt = page_table + (int64_t)seq_slot[seq] * max_blocks;
         float qv[NPL];
         load_q(qv, row);
@@ -280,7 +315,7 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
 #pragma unroll
   for (int r = 0; r < AP_ROWS; ++r) {
     load_q(qv[r], row0 + r);
-    first[r] = window > 0 ? max(0, p0 + r + 1 - window) : 0;
+    first[r] = ap_first(p0 + r, window, chunk);
     total[r].m = -INFINITY;
     total[r].l = 0.f;
 #pragma unroll
@@ -345,7 +380,7 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
 template <typename T, int NPL>
 __global__ __launch_bounds__(256) void attention_plain_join_kernel(
     T* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ positions,
-    const int32_t* __restrict__ row_seq, int H, int hd, int window, int pages) {
+    const int32_t* __restrict__ row_seq, int H, int hd, int window, int chunk, int pages, ApExtras ex) {
   const int lane = threadIdx.x & (HE_WAVE - 1);
   const int h = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int64_t row = blockIdx.x;
@@ -357,9 +392,10 @@ __global__ __launch_bounds__(256) void attention_plain_join_kernel(
   total.l = 0.f;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) total.acc[i] = 0.f;
+  float gf = 1.f;
   if (row_seq[row] >= 0) {
     const int p = positions[row];
-    const int first = window > 0 ? max(0, p + 1 - window) : 0;
+    const int first = ap_first(p, window, chunk);
     const int count = (p >> HE_PAGE_SHIFT) - (first >> HE_PAGE_SHIFT) + 1;
     if (count > pages) {
       // the caller's bound on the keys was too low: no part of the result may pass for one
@@ -390,29 +426,36 @@ __global__ __launch_bounds__(256) void attention_plain_join_kernel(
       for (int u = 0; u < AHEAD; ++u)
         if (z0 + u < count) ap_join(total, part[u]);
     }
+    gf = ap_finish<T, NPL>(total, ex, row, h);
   }
   const float inv = total.l > 0.f ? 1.f / total.l : 0.f;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     const int d = lane + i * HE_WAVE;
-    if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
+    if (i < npl && d < hd) o[d] = from_float<T>(ex.gate ? total.acc[i] * inv * gf : total.acc[i] * inv);
   }
 }
 
 // Pages a query of this step has at most (what a split launch needs room for), given the most keys
 // a sequence holds after the step.
-static int ap_pages(int most_keys, int window) {
+// reach: the most keys a query sees (its window, or its chunk; 0: all before it)
+static int ap_pages(int most_keys, int reach) {
   int pages = (most_keys + HE_PAGE_TOKENS - 1) / HE_PAGE_TOKENS;
-  if (window > 0) pages = min(pages, (window + HE_PAGE_TOKENS - 2) / HE_PAGE_TOKENS + 1);
+  if (reach > 0) pages = min(pages, (reach + HE_PAGE_TOKENS - 2) / HE_PAGE_TOKENS + 1);
   return max(pages, 1);
+}
+static int ap_reach(int window, int chunk) {
+  if (window > 0 && chunk > 0) return min(window, chunk);
+  return window > 0 ? window : max(chunk, 0);
 }
 
 // Floats of workspace with which the step's attention runs page by page in parallel (0: one
 // wavefront per query and head walks the pages itself; that is the better launch for a step with
 // many queries).
-extern "C" int64_t he_attention_plain_workspace_floats(int rows, int H, int hd, int most_keys, int window) {
+extern "C" int64_t he_attention_plain_workspace_floats(int rows, int H, int hd, int most_keys, int window,
+                                                       int chunk) {
   if (rows <= 0 || H <= 0 || hd <= 0 || most_keys <= 0) return 0;
-  const int pages = ap_pages(most_keys, window);
+  const int pages = ap_pages(most_keys, ap_reach(window, chunk));
   if (pages < 2 || (int64_t)rows * H > 8 * he_cus()) return 0;
   return (int64_t)rows * H * pages * (hd + 2);
 }
@@ -420,19 +463,23 @@ extern "C" int64_t he_attention_plain_workspace_floats(int rows, int H, int hd, 
 extern "C" int he_attention_plain(void* out, const void* q, const void* kpool, const void* vpool,
                                   const void* positions, const void* row_seq, const void* seq_slot,
                                   const void* page_table, int max_blocks, int num_pages, int rows,
-                                  int H, int KVH, int hd, int window, float scale, int dtype,
-                                  int most_keys, void* workspace_f32, int64_t workspace_floats,
-                                  void* stream) {
+                                  int H, int KVH, int hd, int window, int chunk, float scale,
+                                  const void* sinks, int sinks_dtype, const void* gate,
+                                  int64_t gate_stride, int dtype, int most_keys, void* workspace_f32,
+                                  int64_t workspace_floats, void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0, "he_attention_plain: bad sizes");
   HE_REQUIRE(H % KVH == 0, "he_attention_plain: heads %d not a multiple of kv heads %d", H, KVH);
   HE_REQUIRE(hd <= AP_MAX_PER_LANE * HE_WAVE, "he_attention_plain: head_dim %d above %d", hd,
              AP_MAX_PER_LANE * HE_WAVE);
   HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_attention_plain: unknown dtype %d", dtype);
+  HE_REQUIRE(sinks == nullptr || sinks_dtype == HE_BF16 || sinks_dtype == HE_F32,
+             "he_attention_plain: unknown dtype %d of the sinks", sinks_dtype);
   if (rows == 0) return 0;
+  const ApExtras ex = {sinks, sinks_dtype, gate, gate_stride};
   // page by page in parallel when the caller brought room for it (the same bits either way)
-  const int64_t need = he_attention_plain_workspace_floats(rows, H, hd, most_keys, window);
+  const int64_t need = he_attention_plain_workspace_floats(rows, H, hd, most_keys, window, chunk);
   const bool split = need > 0 && workspace_f32 != nullptr && workspace_floats >= need;
-  const int pages = split ? ap_pages(most_keys, window) : 1;
+  const int pages = split ? ap_pages(most_keys, ap_reach(window, chunk)) : 1;
   HE_REQUIRE(pages <= 65535, "he_attention_plain: %d pages of keys are too many for one launch", pages);
   dim3 grid(rows, (H + 3) / 4, pages);
   float* ws = (float*)workspace_f32;
@@ -441,10 +488,10 @@ extern "C" int he_attention_plain(void* out, const void* q, const void* kpool, c
   attention_plain_kernel<T, NPL><<<grid, 256, 0, s>>>(                                         \
       (T*)out, ws, (const T*)q, (const T*)kpool, (const T*)vpool, (const int32_t*)positions,   \
       (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table,           \
-      max_blocks, num_pages, H, KVH, hd, window, scale)
+      max_blocks, num_pages, H, KVH, hd, window, chunk, scale, ex)
 #define AP_JOIN(T, NPL)                                                                        \
   attention_plain_join_kernel<T, NPL><<<dim3(rows, (H + 3) / 4), 256, 0, s>>>(                 \
-      (T*)out, ws, (const int32_t*)positions, (const int32_t*)row_seq, H, hd, window, pages)
+      (T*)out, ws, (const int32_t*)positions, (const int32_t*)row_seq, H, hd, window, chunk, pages, ex)
   const int npl = (hd + HE_WAVE - 1) / HE_WAVE;   // elements a lane holds: 1, 2, up to 4, up to 8
 #define AP_BY_SIZE(WHAT)                                  \
   if (dtype == HE_BF16) {                                 \
@@ -462,7 +509,7 @@ extern "C" int he_attention_plain(void* out, const void* q, const void* kpool, c
   attention_plain_rows_kernel<T, NPL><<<dim3((rows + AP_ROWS - 1) / AP_ROWS, (H + 3) / 4), 256, 0, s>>>(   \
       (T*)out, (const T*)q, (const T*)kpool, (const T*)vpool, (const int32_t*)positions,               \
       (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,       \
-      num_pages, rows, H, KVH, hd, window, scale)
+      num_pages, rows, H, KVH, hd, window, chunk, scale, ex)
   if (!split && rows >= 64) {      // a step of many queries: four neighbours a wavefront share their keys
     AP_BY_SIZE(AP_ROWS_LAUNCH)
     return he_check_launch("he_attention_plain");

@@ -177,6 +177,20 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return total;
 }
 
+// A gated activation's constants: out = g' * sigmoid(alpha g') * (u' + shift) with g' = min(g, limit),
+// u' = clamp(u, -limit, limit) (limit +inf: unbounded). CLAMPED false is SiLU(g) * u, written as it
+// always was (the constants are then not read).
+struct GatedAct {
+  float alpha, limit, shift;
+};
+template <bool CLAMPED>
+__device__ __forceinline__ float he_gated_act(float g, float u, const GatedAct& a) {
+  if (!CLAMPED) return g / (1.f + expf(-g)) * u;
+  g = fminf(g, a.limit);
+  u = fminf(fmaxf(u, -a.limit), a.limit);
+  return g / (1.f + expf(-a.alpha * g)) * (u + a.shift);
+}
+
 // ---- error channel -------------------------------------------------------
 void he_set_error(const char* fmt, ...);
 int he_check_launch(const char* what);

@@ -4,11 +4,11 @@
 #include "common.h"
 #include "hector_kernels.h"
 
-// out[t, :] = table[ids[t], :] as fp32; an id outside [0, V) gives a zero row
-// (reference: kernels/linear.cu:36-69).
+// out[t, :] = table[ids[t], :] * scale as fp32 (scale 1: the row as it is); an id outside
+// [0, V) gives a zero row (reference: kernels/linear.cu:36-69).
 template <typename T>
 __global__ void embedding_kernel(float* __restrict__ out, const T* __restrict__ table,
-                                 const int32_t* __restrict__ ids, int D, int V) {
+                                 const int32_t* __restrict__ ids, int D, int V, float scale) {
   const int64_t t = blockIdx.x;
   const int id = ids[t];
   float* o = out + t * (int64_t)D;
@@ -25,29 +25,29 @@ __global__ void embedding_kernel(float* __restrict__ out, const T* __restrict__ 
       float f[8];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        f[2 * j] = __uint_as_float(w[j] << 16);
-        f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        f[2 * j] = __uint_as_float(w[j] << 16) * scale;
+        f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u) * scale;
       }
       *reinterpret_cast<float4*>(o + i) = make_float4(f[0], f[1], f[2], f[3]);
       *reinterpret_cast<float4*>(o + i + 4) = make_float4(f[4], f[5], f[6], f[7]);
     }
     return;
   }
-  for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = to_float(row[i]);
+  for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = to_float(row[i]) * scale;
 }
 
 extern "C" int he_embedding(void* out_f32, const void* table, const void* ids, int rows, int D,
-                            int V, int table_dtype, void* stream) {
+                            int V, int table_dtype, float scale, void* stream) {
   HE_REQUIRE(rows >= 0 && D > 0 && V > 0, "he_embedding: bad sizes rows=%d D=%d V=%d", rows, D, V);
   if (rows == 0) return 0;
   const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
   hipStream_t s = (hipStream_t)stream;
   if (table_dtype == HE_BF16)
     embedding_kernel<bf16_t><<<rows, threads, 0, s>>>((float*)out_f32, (const bf16_t*)table,
-                                                      (const int32_t*)ids, D, V);
+                                                      (const int32_t*)ids, D, V, scale);
   else if (table_dtype == HE_F32)
     embedding_kernel<float><<<rows, threads, 0, s>>>((float*)out_f32, (const float*)table,
-                                                     (const int32_t*)ids, D, V);
+                                                     (const int32_t*)ids, D, V, scale);
   else
     HE_REQUIRE(false, "he_embedding: unknown dtype %d", table_dtype);
   return he_check_launch("he_embedding");
@@ -81,17 +81,17 @@ extern "C" int he_gather_rows_f32(void* out, const void* src, const void* rows, 
   return he_check_launch("he_gather_rows_f32");
 }
 
-// resid[r, :] += delta[r, :], the residual sum in fp32.
+// resid[r, :] += scale * delta[r, :], the residual sum in fp32 (scale 1: the plain sum).
 template <typename T>
 __global__ void residual_add_kernel(float* __restrict__ resid, const T* __restrict__ delta,
-                                    int64_t n) {
+                                    int64_t n, float scale) {
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (; i < n; i += stride) resid[i] += to_float(delta[i]);
+  for (; i < n; i += stride) resid[i] += scale * to_float(delta[i]);
 }
 
 extern "C" int he_residual_add(void* resid_f32, const void* delta, int64_t n, int delta_dtype,
-                               void* stream) {
+                               float scale, void* stream) {
   HE_REQUIRE(n >= 0, "he_residual_add: bad size");
   if (n == 0) return 0;
   int64_t blocks = (n + 255) / 256;
@@ -99,10 +99,10 @@ extern "C" int he_residual_add(void* resid_f32, const void* delta, int64_t n, in
   hipStream_t s = (hipStream_t)stream;
   if (delta_dtype == HE_BF16)
     residual_add_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((float*)resid_f32,
-                                                            (const bf16_t*)delta, n);
+                                                            (const bf16_t*)delta, n, scale);
   else if (delta_dtype == HE_F32)
     residual_add_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)resid_f32, (const float*)delta,
-                                                           n);
+                                                           n, scale);
   else
     HE_REQUIRE(false, "he_residual_add: unknown dtype %d", delta_dtype);
   return he_check_launch("he_residual_add");
@@ -110,14 +110,15 @@ extern "C" int he_residual_add(void* resid_f32, const void* delta, int64_t n, in
 
 // out[r, i] = silu(gate[r, i]) * up[r, i] with x = [rows, 2I],
 // silu(z) = z / (1 + exp(-z)) in fp32 (reference: kernels/activations.cu:19-21,183-198).
+// CLAMPED: the gated activation with its constants (common.h: he_gated_act).
 // Column layout of x: gate then up (x[r, i], x[r, I + i]); or interleaved, as the
 // fused gate||up weight of the MFMA path lays its rows out: gate i at column 2i,
 // its up at 2i + 1.
 // With splits > 0, x is the fp32 K slices [splits][rows][2I] of the gate||up product,
 // added here in the order of the slice index.
-template <typename T, typename TI>
+template <typename T, typename TI, bool CLAMPED>
 __global__ void silu_mul_kernel(T* __restrict__ out, const TI* __restrict__ x, int64_t rows,
-                                int I, int interleaved, int splits) {
+                                int I, int interleaved, int splits, GatedAct act) {
   const int64_t n = rows * (int64_t)I;
   const int64_t split_stride = rows * 2 * (int64_t)I;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
@@ -133,15 +134,16 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const TI* __restrict__ x, i
       g += to_float(row[s * split_stride + gc]);
       u += to_float(row[s * split_stride + uc]);
     }
-    const float y = g / (1.f + expf(-g)) * u;
+    const float y = he_gated_act<CLAMPED>(g, u, act);
     out[i] = from_float<T>(y);
   }
 }
 
 // bf16, eight outputs per thread, I a multiple of 8: eight consecutive gates and their ups are
 // two runs of 16 bytes, or, interleaved, one run of 32 bytes of (gate, up) pairs.
+template <bool CLAMPED>
 __global__ void silu_mul_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x,
-                                    int64_t rows, int I, int interleaved) {
+                                    int64_t rows, int I, int interleaved, GatedAct act) {
   const int64_t n8 = rows * (int64_t)(I >> 3);
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -159,7 +161,7 @@ __global__ void silu_mul_vec_kernel(uint16_t* __restrict__ out, const uint16_t* 
       for (int j = 0; j < 4; ++j) {
         const float g0 = __uint_as_float(w[2 * j] << 16), u0 = __uint_as_float(w[2 * j] & 0xffff0000u);
         const float g1 = __uint_as_float(w[2 * j + 1] << 16), u1 = __uint_as_float(w[2 * j + 1] & 0xffff0000u);
-        o[j] = pack2_bf16(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+        o[j] = pack2_bf16(he_gated_act<CLAMPED>(g0, u0, act), he_gated_act<CLAMPED>(g1, u1, act));
       }
     } else {
       const uint4 g4 = *reinterpret_cast<const uint4*>(row + c);
@@ -169,43 +171,62 @@ __global__ void silu_mul_vec_kernel(uint16_t* __restrict__ out, const uint16_t* 
       for (int j = 0; j < 4; ++j) {
         const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
         const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-        o[j] = pack2_bf16(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+        o[j] = pack2_bf16(he_gated_act<CLAMPED>(g0, u0, act), he_gated_act<CLAMPED>(g1, u1, act));
       }
     }
     *reinterpret_cast<uint4*>(out + r * (int64_t)I + c) = make_uint4(o[0], o[1], o[2], o[3]);
   }
 }
 
-extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int interleaved,
-                           int splits, int dtype, void* stream) {
-  HE_REQUIRE(rows >= 0 && I > 0, "he_silu_mul: bad sizes rows=%d I=%d", rows, I);
-  HE_REQUIRE(splits >= 0 && splits <= 64, "he_silu_mul: bad slice count %d", splits);
-  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_silu_mul: unknown dtype %d", dtype);
-  if (rows == 0) return 0;
+template <bool CLAMPED>
+static int gated_act_launch(void* out, const void* gate_up, int rows, int I, int interleaved, int splits,
+                            int dtype, GatedAct act, hipStream_t s) {
   const int64_t n = (int64_t)rows * I;
   int64_t blocks = (n + 255) / 256;
   if (blocks > 65535 * 4) blocks = 65535 * 4;
-  hipStream_t s = (hipStream_t)stream;
   if (splits == 0 && dtype == HE_BF16 && (I & 7) == 0 &&
       ((((uintptr_t)out) | ((uintptr_t)gate_up)) & 15) == 0) {
     const int64_t n8 = n >> 3;
     int64_t vb = (n8 + 255) / 256;
     if (vb > 65535 * 4) vb = 65535 * 4;
-    silu_mul_vec_kernel<<<(int)vb, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)gate_up, rows, I,
-                                                interleaved);
+    silu_mul_vec_kernel<CLAMPED><<<(int)vb, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)gate_up, rows, I,
+                                                         interleaved, act);
   } else if (splits > 0) {  // fp32 partial sums in
     if (dtype == HE_BF16)
-      silu_mul_kernel<bf16_t, float><<<(int)blocks, 256, 0, s>>>(
-          (bf16_t*)out, (const float*)gate_up, rows, I, interleaved, splits);
+      silu_mul_kernel<bf16_t, float, CLAMPED><<<(int)blocks, 256, 0, s>>>(
+          (bf16_t*)out, (const float*)gate_up, rows, I, interleaved, splits, act);
     else
-      silu_mul_kernel<float, float><<<(int)blocks, 256, 0, s>>>(
-          (float*)out, (const float*)gate_up, rows, I, interleaved, splits);
+      silu_mul_kernel<float, float, CLAMPED><<<(int)blocks, 256, 0, s>>>(
+          (float*)out, (const float*)gate_up, rows, I, interleaved, splits, act);
   } else if (dtype == HE_BF16) {
-    silu_mul_kernel<bf16_t, bf16_t><<<(int)blocks, 256, 0, s>>>(
-        (bf16_t*)out, (const bf16_t*)gate_up, rows, I, interleaved, 1);
+    silu_mul_kernel<bf16_t, bf16_t, CLAMPED><<<(int)blocks, 256, 0, s>>>(
+        (bf16_t*)out, (const bf16_t*)gate_up, rows, I, interleaved, 1, act);
   } else {
-    silu_mul_kernel<float, float><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)gate_up,
-                                                              rows, I, interleaved, 1);
+    silu_mul_kernel<float, float, CLAMPED><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)gate_up,
+                                                                       rows, I, interleaved, 1, act);
   }
-  return he_check_launch("he_silu_mul");
+  return he_check_launch("he_gated_act");
+}
+
+// out = act(gate) * up over gate||up columns as he_silu_mul takes them, with
+// gate' = min(gate, limit), up' = clamp(up, -limit, limit) (limit <= 0: neither is bounded),
+// out = gate' * sigmoid(alpha * gate') * (up' + up_shift). alpha 1, no limit and no shift is SiLU(gate) * up.
+extern "C" int he_gated_act(void* out, const void* gate_up, int rows, int I, int interleaved, int splits,
+                            int dtype, float alpha, float limit, float up_shift, void* stream) {
+  HE_REQUIRE(rows >= 0 && I > 0, "he_gated_act: bad sizes rows=%d I=%d", rows, I);
+  HE_REQUIRE(splits >= 0 && splits <= 64, "he_gated_act: bad slice count %d", splits);
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_gated_act: unknown dtype %d", dtype);
+  if (rows == 0) return 0;
+  GatedAct act;
+  act.alpha = alpha;
+  act.limit = limit > 0.f ? limit : INFINITY;
+  act.shift = up_shift;
+  if (alpha == 1.f && !(limit > 0.f) && up_shift == 0.f)
+    return gated_act_launch<false>(out, gate_up, rows, I, interleaved, splits, dtype, act, (hipStream_t)stream);
+  return gated_act_launch<true>(out, gate_up, rows, I, interleaved, splits, dtype, act, (hipStream_t)stream);
+}
+
+extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int interleaved,
+                           int splits, int dtype, void* stream) {
+  return he_gated_act(out, gate_up, rows, I, interleaved, splits, dtype, 1.f, 0.f, 0.f, stream);
 }

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 20
+#define HE_ABI_VERSION 21
 
 #ifdef __cplusplus
 extern "C" {
@@ -26,19 +26,33 @@ int he_fill_random_integers(void* out_i32, int64_t n, uint64_t key, int64_t high
 int he_cast(void* out, const void* in, int64_t n, int in_dtype, int out_dtype, void* stream);
 
 // ---- row-wise ------------------------------------------------------------
+// out[t, :] = table[ids[t], :] * scale in fp32.
 int he_embedding(void* out_f32, const void* table, const void* ids, int rows, int D, int V,
-                 int table_dtype, void* stream);
+                 int table_dtype, float scale, void* stream);
 int he_gather_rows_f32(void* out, const void* src, const void* rows, int n_out, int D, int n_src,
                        void* stream);
-int he_residual_add(void* resid_f32, const void* delta, int64_t n, int delta_dtype, void* stream);
+// resid += scale * delta.
+int he_residual_add(void* resid_f32, const void* delta, int64_t n, int delta_dtype, float scale,
+                    void* stream);
 // splits > 0: gate_up is fp32 [splits][rows][2I], the K slices of the product.
 int he_silu_mul(void* out, const void* gate_up, int rows, int I, int interleaved, int splits,
                 int dtype, void* stream);
+// The same columns through a gated activation with constants: gate' = min(gate, limit),
+// up' = clamp(up, -limit, limit) (limit <= 0: unbounded), out = gate' * sigmoid(alpha * gate') *
+// (up' + up_shift). alpha 1 without limit and shift is he_silu_mul.
+int he_gated_act(void* out, const void* gate_up, int rows, int I, int interleaved, int splits,
+                 int dtype, float alpha, float limit, float up_shift, void* stream);
 
 // ---- norms ---------------------------------------------------------------
 // resid (fp32, in place) += delta (may be null); out (may be null) = rmsnorm(resid) * weight.
 int he_add_rmsnorm(void* resid_f32, const void* delta, const void* weight, void* out, int rows, int D,
                    float eps, int act_dtype, int w_dtype, void* stream);
+// Dynamic Tanh where a norm would stand: resid (fp32, in place) += delta_scale * delta (may be null);
+// out (may be null) = tanh(alpha * resid) * weight + bias, alpha a stored scalar (device pointer),
+// weight and bias vectors [D], all three of w_dtype.
+int he_add_dyt(void* resid_f32, const void* delta, float delta_scale, const void* weight,
+               const void* bias, const void* alpha, void* out, int rows, int D, int act_dtype,
+               int w_dtype, void* stream);
 int he_rmsnorm_rows(void* out, const void* x, const void* weight, int rows, int D,
                     int64_t x_stride, int64_t out_stride, float eps, int dtype, int w_dtype,
                     void* stream);
@@ -108,7 +122,12 @@ int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in, c
                       const void* v_bias, int bias_dtype, const void* positions,
                       const void* row_seq, const void* seq_slot, const void* page_table,
                       int max_blocks, int num_pages, const void* inv_freq, int rotary_dim, int rows,
-                      int H, int KVH, int hd, int dtype, void* stream);
+                      int H, int KVH, int hd, int hd_in, int vd_in, int interleaved, float mscale,
+                      int dtype, void* stream);
+// hd: head size of q_out and of the cache pages. hd_in, vd_in (0: hd): head sizes of the q/k rows and
+// of the v rows that come in (at most hd; q_out is padded with zeros, the pages keep their zeros).
+// interleaved: frequency i turns the pair (2i, 2i + 1), not (i, i + rotary_dim / 2). mscale multiplies
+// cos and sin.
 
 // ---- attention over the paged cache ----------------------------------------
 // he_attention_plain: fp32 sums in one fixed order per (query, head): page by page (64 positions),
@@ -116,12 +135,18 @@ int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in, c
 // position. most_keys: no sequence holds more keys after the step. With a workspace of
 // he_attention_plain_workspace_floats floats (0 for a step of many queries) the pages of a query
 // run in parallel and a second kernel joins them; the result is the same bit for bit.
-int64_t he_attention_plain_workspace_floats(int rows, int H, int hd, int most_keys, int window);
+// chunk > 0: a query sees no key before the start of its own chunk of that many positions (counted
+// from position 0). sinks (or null): one number a head that joins the softmax's denominator as
+// exp(sink), without a value. gate (or null): gate[row * gate_stride + h], in the activation dtype;
+// the head's output is multiplied by sigmoid(gate).
+int64_t he_attention_plain_workspace_floats(int rows, int H, int hd, int most_keys, int window,
+                                            int chunk);
 int he_attention_plain(void* out, const void* q, const void* kpool, const void* vpool,
                        const void* positions, const void* row_seq, const void* seq_slot,
                        const void* page_table, int max_blocks, int num_pages, int rows, int H,
-                       int KVH, int hd, int window, float scale, int dtype, int most_keys,
-                       void* workspace_f32, int64_t workspace_floats, void* stream);
+                       int KVH, int hd, int window, int chunk, float scale, const void* sinks,
+                       int sinks_dtype, const void* gate, int64_t gate_stride, int dtype,
+                       int most_keys, void* workspace_f32, int64_t workspace_floats, void* stream);
 // bf16, one query row per sequence (decode): split over the keys, then merged.
 int he_attention_decode_bf16(void* out, const void* q, const void* kpool, const void* vpool,
                              const void* positions, const void* row_seq, const void* seq_slot,

@@ -288,3 +288,84 @@ extern "C" int he_scale_rows_bf16(void* out, const void* x, const void* partials
       (uint16_t*)out, (const uint16_t*)x, (const float*)partials, count, D, eps, x_pieces);
   return he_check_launch("he_scale_rows_bf16");
 }
+
+// Dynamic Tanh in place of a norm: y = tanh(alpha * r) * w + b with a scalar alpha and vectors w, b;
+// it reduces nothing over the row, so it is one pass over the elements. As the fused add + RMS norm
+// above, it first adds the pending branch output: r = resid + delta_scale * delta (fp32, stored
+// back as the new residual). alpha is read from device memory (a stored tensor of one element).
+template <typename TD, typename TO, typename TW, int VEC>
+__global__ void add_dyt_kernel(float* __restrict__ resid, const TD* __restrict__ delta, float delta_scale,
+                               const TW* __restrict__ w, const TW* __restrict__ b,
+                               const TW* __restrict__ alpha_p, TO* __restrict__ out, int64_t n, int D) {
+  const float alpha = to_float(alpha_p[0]);
+  int64_t i = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) * VEC;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x * VEC;
+  for (; i < n; i += stride) {
+    const int c = (int)(i % D);
+    float v[VEC], a[VEC], g[VEC], s[VEC];
+    if constexpr (VEC == 4) {
+      load4(resid + i, v);
+      if (delta) load4(delta + i, a);
+      if (out) {
+        load4(w + c, g);
+        load4(b + c, s);
+      }
+    } else {
+      v[0] = resid[i];
+      if (delta) a[0] = to_float(delta[i]);
+      if (out) g[0] = to_float(w[c]), s[0] = to_float(b[c]);
+    }
+    if (delta) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = fmaf(delta_scale, a[j], v[j]);
+      if constexpr (VEC == 4) store4(resid + i, v);
+      else resid[i] = v[0];
+    }
+    if (out) {
+      float y[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) y[j] = fmaf(tanhf(alpha * v[j]), g[j], s[j]);
+      if constexpr (VEC == 4) store4(out + i, y);
+      else out[i] = from_float<TO>(y[0]);
+    }
+  }
+}
+
+template <typename TD, typename TO, typename TW>
+static void launch_add_dyt(float* resid, const void* delta, float delta_scale, const void* w, const void* b,
+                           const void* alpha, void* out, int rows, int D, hipStream_t s) {
+  const int64_t n = (int64_t)rows * D;
+  const bool vec = (D & 3) == 0 && ((((uintptr_t)resid) | ((uintptr_t)delta) | ((uintptr_t)w) | ((uintptr_t)b) |
+                                     ((uintptr_t)out)) & 15) == 0;
+  const int64_t items = vec ? n / 4 : n;
+  int64_t blocks = (items + 255) / 256;
+  if (blocks > 65535 * 16) blocks = 65535 * 16;
+  if (vec)
+    add_dyt_kernel<TD, TO, TW, 4><<<(unsigned)blocks, 256, 0, s>>>(resid, (const TD*)delta, delta_scale, (const TW*)w,
+                                                                   (const TW*)b, (const TW*)alpha, (TO*)out, n, D);
+  else
+    add_dyt_kernel<TD, TO, TW, 1><<<(unsigned)blocks, 256, 0, s>>>(resid, (const TD*)delta, delta_scale, (const TW*)w,
+                                                                   (const TW*)b, (const TW*)alpha, (TO*)out, n, D);
+}
+
+extern "C" int he_add_dyt(void* resid_f32, const void* delta, float delta_scale, const void* weight,
+                          const void* bias, const void* alpha, void* out, int rows, int D, int act_dtype,
+                          int w_dtype, void* stream) {
+  HE_REQUIRE(rows >= 0 && D > 0, "he_add_dyt: bad sizes rows=%d D=%d", rows, D);
+  HE_REQUIRE(w_dtype == HE_F32 || w_dtype == HE_BF16, "he_add_dyt: bad parameter dtype");
+  HE_REQUIRE(act_dtype == HE_F32 || act_dtype == HE_BF16, "he_add_dyt: unknown dtype %d", act_dtype);
+  HE_REQUIRE(out == nullptr || (weight && bias && alpha), "he_add_dyt: weight, bias and alpha are needed");
+  if (rows == 0 || (delta == nullptr && out == nullptr)) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  float* r = (float*)resid_f32;
+#define DYT(TD, TO, TW) launch_add_dyt<TD, TO, TW>(r, delta, delta_scale, weight, bias, alpha, out, rows, D, s)
+  if (act_dtype == HE_BF16) {
+    if (w_dtype == HE_BF16) DYT(bf16_t, bf16_t, bf16_t);
+    else DYT(bf16_t, bf16_t, float);
+  } else {
+    if (w_dtype == HE_BF16) DYT(float, float, bf16_t);
+    else DYT(float, float, float);
+  }
+#undef DYT
+  return he_check_launch("he_add_dyt");
+}

@@ -13,6 +13,11 @@
 
 #define ROPE_MAX_HALF 256
 
+// hd: the head size of q_out and of the cache pages; hd_in <= hd, vd_in <= hd: the head sizes of the
+// projected q/k and v rows (a mixer whose keys and values differ in width keeps both in pages of
+// the wider one: q_out's dims from hd_in on are written as zeros, those of the pages are never
+// written and stay the zeros the pools were made with). interleaved: the pair of frequency i is
+// (2i, 2i + 1) instead of (i, i + r/2). mscale multiplies cos and sin (1: a pure rotation).
 template <typename T, typename TI>
 __global__ void qkv_rope_cache_kernel(
     T* __restrict__ q_out, T* __restrict__ kpool, T* __restrict__ vpool,
@@ -21,7 +26,8 @@ __global__ void qkv_rope_cache_kernel(
     const void* __restrict__ v_bias, int bias_dtype, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ page_table, int max_blocks, int num_pages,
-    const float* __restrict__ inv_freq, int rotary_dim, int H, int KVH, int hd) {
+    const float* __restrict__ inv_freq, int rotary_dim, int H, int KVH, int hd, int hd_in, int vd_in,
+    int interleaved, float mscale) {
   __shared__ float cs[2][ROPE_MAX_HALF];
   const int64_t row = blockIdx.x;
   const int seq = row_seq[row];
@@ -32,10 +38,13 @@ __global__ void qkv_rope_cache_kernel(
     const float a = (float)pos * inv_freq[i];
     float sn, c;
     sincos_angle(a, &sn, &c);
-    cs[0][i] = c;
-    cs[1][i] = sn;
+    cs[0][i] = c * mscale;
+    cs[1][i] = sn * mscale;
   }
   __syncthreads();
+  // the two dims of pair j
+  const int pair_step = interleaved ? 1 : half;
+  const int pair_mul = interleaved ? 2 : 1;
 
   // ---- q: rotate and store densely
   {
@@ -45,22 +54,26 @@ __global__ void qkv_rope_cache_kernel(
     for (int it = threadIdx.x; it < H * per_head; it += blockDim.x) {
       const int h = it / per_head;
       const int j = it - h * per_head;
-      const int base = h * hd;
+      const int base = h * hd_in, obase = h * hd;
       if (j < half) {
-        float x0 = to_float((in + base + j)[0]);
-        float x1 = to_float((in + base + j + half)[0]);
+        const int d0 = pair_mul * j, d1 = d0 + pair_step;
+        float x0 = to_float((in + base + d0)[0]);
+        float x1 = to_float((in + base + d1)[0]);
         if (q_bias) {
-          x0 += load_param(q_bias, base + j, bias_dtype);
-          x1 += load_param(q_bias, base + j + half, bias_dtype);
+          x0 += load_param(q_bias, base + d0, bias_dtype);
+          x1 += load_param(q_bias, base + d1, bias_dtype);
         }
         const float c = cs[0][j], sn = cs[1][j];
-        out[base + j] = from_float<T>(x0 * c - x1 * sn);
-        out[base + j + half] = from_float<T>(x0 * sn + x1 * c);
+        out[obase + d0] = from_float<T>(x0 * c - x1 * sn);
+        out[obase + d1] = from_float<T>(x0 * sn + x1 * c);
       } else {
         const int d = rotary_dim + (j - half);
-        float x = to_float((in + base + d)[0]);
-        if (q_bias) x += load_param(q_bias, base + d, bias_dtype);
-        out[base + d] = from_float<T>(x);
+        float x = 0.f;
+        if (d < hd_in) {
+          x = to_float((in + base + d)[0]);
+          if (q_bias) x += load_param(q_bias, base + d, bias_dtype);
+        }
+        out[obase + d] = from_float<T>(x);
       }
     }
   }
@@ -73,23 +86,24 @@ __global__ void qkv_rope_cache_kernel(
   // ---- k: rotate and scatter
   {
     const TI* in = k_in + row * in_stride;
-    const int per_head = half + (hd - rotary_dim);
+    const int per_head = half + (hd_in - rotary_dim);
     for (int it = threadIdx.x; it < KVH * per_head; it += blockDim.x) {
       const int h = it / per_head;
       const int j = it - h * per_head;
-      const int base = h * hd;
+      const int base = h * hd_in;
       T* out = kpool + ((int64_t)page * KVH + h) * he_k_page_elems(hd);   // the page, in operand order
       const int KS = he_k_steps(hd);
       if (j < half) {
-        float x0 = to_float((in + base + j)[0]);
-        float x1 = to_float((in + base + j + half)[0]);
+        const int d0 = pair_mul * j, d1 = d0 + pair_step;
+        float x0 = to_float((in + base + d0)[0]);
+        float x1 = to_float((in + base + d1)[0]);
         if (k_bias) {
-          x0 += load_param(k_bias, base + j, bias_dtype);
-          x1 += load_param(k_bias, base + j + half, bias_dtype);
+          x0 += load_param(k_bias, base + d0, bias_dtype);
+          x1 += load_param(k_bias, base + d1, bias_dtype);
         }
         const float c = cs[0][j], sn = cs[1][j];
-        out[he_k_index(off, j, KS)] = from_float<T>(x0 * c - x1 * sn);
-        out[he_k_index(off, j + half, KS)] = from_float<T>(x0 * sn + x1 * c);
+        out[he_k_index(off, d0, KS)] = from_float<T>(x0 * c - x1 * sn);
+        out[he_k_index(off, d1, KS)] = from_float<T>(x0 * sn + x1 * c);
       } else {
         const int d = rotary_dim + (j - half);
         float x = to_float((in + base + d)[0]);
@@ -101,9 +115,9 @@ __global__ void qkv_rope_cache_kernel(
   // ---- v: bias and scatter
   {
     const TI* in = v_in + row * in_stride;
-    for (int it = threadIdx.x; it < KVH * hd; it += blockDim.x) {
-      const int h = it / hd;
-      const int d = it - h * hd;
+    for (int it = threadIdx.x; it < KVH * vd_in; it += blockDim.x) {
+      const int h = it / vd_in;
+      const int d = it - h * vd_in;
       float x = to_float((in + it)[0]);
       if (v_bias) x += load_param(v_bias, it, bias_dtype);
       vpool[((int64_t)page * KVH + h) * he_v_page_elems(hd) + he_v_index(off, d, he_v_tiles(hd))] =
@@ -305,11 +319,16 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
                                  int bias_dtype, const void* positions, const void* row_seq,
                                  const void* seq_slot, const void* page_table, int max_blocks,
                                  int num_pages, const void* inv_freq, int rotary_dim, int rows,
-                                 int H, int KVH, int hd, int dtype, void* stream) {
+                                 int H, int KVH, int hd, int hd_in, int vd_in, int interleaved,
+                                 float mscale, int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH >= 0 && hd > 0, "he_qkv_rope_cache: bad sizes");
-  HE_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && (rotary_dim & 1) == 0,
+  if (hd_in <= 0) hd_in = hd;
+  if (vd_in <= 0) vd_in = hd;
+  HE_REQUIRE(hd_in <= hd && vd_in <= hd,
+             "he_qkv_rope_cache: the rows' head sizes %d and %d exceed the pages' %d", hd_in, vd_in, hd);
+  HE_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd_in && (rotary_dim & 1) == 0,
              "he_qkv_rope_cache: rotary_dim %d must be even and at most head_dim %d", rotary_dim,
-             hd);
+             hd_in);
   HE_REQUIRE(rotary_dim / 2 <= ROPE_MAX_HALF, "he_qkv_rope_cache: rotary_dim %d above %d",
              rotary_dim, 2 * ROPE_MAX_HALF);
   HE_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "he_qkv_rope_cache: missing inv_freq");
@@ -326,8 +345,8 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
       in_stride, q_bias, k_bias, v_bias, bias_dtype,                                            \
       (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot,             \
       (const int32_t*)page_table, max_blocks, num_pages, (const float*)inv_freq, rotary_dim, H, \
-      KVH, hd)
-  const bool vec_ok = dtype == HE_BF16 &&
+      KVH, hd, hd_in, vd_in, interleaved, mscale)
+  const bool vec_ok = dtype == HE_BF16 && hd_in == hd && vd_in == hd && !interleaved && mscale == 1.f &&
                       (q_bias == nullptr || bias_dtype == HE_BF16) &&
                       ((rotary_dim >> 1) & 7) == 0 && ((hd - rotary_dim) & 7) == 0 &&
                       (in_stride & 7) == 0 && (hd & 7) == 0 &&

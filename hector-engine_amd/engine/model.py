@@ -86,12 +86,21 @@ class DecoderModel:
         rows = ctx.rows
         resid = self.embedding.forward(ids, rows, ctx)
         stream = ResidualStream(resid, rows)
+        embedded = None
+        if any(entry.add_embedding for entry in self.schedule):
+            # the embedding's output, kept for the runs that start again from it
+            embedded = ctx.alloc((rows, self.spec.hidden_size), torch.float32)
+            embedded.copy_(resid)
         last = len(self.schedule) - 1
         for e, entry in enumerate(self.schedule):
+            if entry.add_embedding:
+                ops.residual_add(stream.materialize(ctx), embedded, rows)
             # the norm that reads the stream after this block: the next block's first, or the
             # final norm when every row's logits are wanted (no gather in between)
             if e < last:
-                ctx.next_norm = self.blocks[self.schedule[e + 1].layer].first_norm()
+                # (a run that first takes the embedding again reads the stream through that sum)
+                ctx.next_norm = None if self.schedule[e + 1].add_embedding else \
+                    self.blocks[self.schedule[e + 1].layer].first_norm()
             else:
                 ctx.next_norm = self.final_norm if (ctx.want_all and n_want == rows) else None
             ctx.scratch.begin_layer()

@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 20
+EXPECTED_ABI = 21
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -26,10 +26,12 @@ _SIGNATURES = {
     "he_fill_random": [c_ptr, c_i64, c_int, ctypes.c_uint64, c_ptr, c_f32, c_f32, c_ptr],
     "he_fill_random_integers": [c_ptr, c_i64, ctypes.c_uint64, c_i64, c_ptr],
     "he_cast": [c_ptr, c_ptr, c_i64, c_int, c_int, c_ptr],
-    "he_embedding": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_ptr],
+    "he_embedding": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_f32, c_ptr],
     "he_gather_rows_f32": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_ptr],
-    "he_residual_add": [c_ptr, c_ptr, c_i64, c_int, c_ptr],
+    "he_residual_add": [c_ptr, c_ptr, c_i64, c_int, c_f32, c_ptr],
     "he_silu_mul": [c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
+    "he_gated_act": [c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_f32, c_ptr],
+    "he_add_dyt": [c_ptr, c_ptr, c_f32, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_ptr],
     "he_add_rmsnorm": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_f32, c_int, c_int, c_ptr],
     "he_rmsnorm_rows": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_i64, c_i64, c_f32, c_int, c_int, c_ptr],
     "he_gemm_plain_workspace_floats": [c_int, c_int, c_int],
@@ -52,10 +54,11 @@ _SIGNATURES = {
                                   c_int, c_int, c_ptr],
     "he_qkv_rope_cache": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr,
                           c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int,
-                          c_int, c_int, c_int, c_int, c_ptr],
-    "he_attention_plain_workspace_floats": [c_int, c_int, c_int, c_int, c_int],
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr],
+    "he_attention_plain_workspace_floats": [c_int, c_int, c_int, c_int, c_int, c_int],
     "he_attention_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_int, c_ptr, c_i64, c_ptr],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_ptr, c_int, c_ptr, c_i64,
+                           c_int, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_decode_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr,
                                  c_i64, c_ptr],

@@ -74,7 +74,8 @@ def cast(out, src) -> None:
 
 
 @_op("embedding")
-def embedding(out_f32, table, ids, rows: int) -> None:
+def embedding(out_f32, table, ids, rows: int, scale: float = 1.0) -> None:
+    """out[t] = table[ids[t]] * scale in fp32."""
     V, D = table.shape
     _need(table, "table")
     _need(out_f32, "out", torch.float32)
@@ -83,7 +84,7 @@ def embedding(out_f32, table, ids, rows: int) -> None:
         raise ValueError("embedding: buffers smaller than the row count")
     L = _lib.load()
     _lib.check(L.he_embedding(out_f32.data_ptr(), table.data_ptr(), ids.data_ptr(), rows, D, V,
-                              dtype_code(table.dtype), _stream()))
+                              dtype_code(table.dtype), float(scale), _stream()))
 
 
 @_op("gather_rows")
@@ -100,7 +101,8 @@ def gather_rows_f32(out, src, rows_idx, n_out: int, n_src: int) -> None:
 
 
 @_op("residual_add")
-def residual_add(resid_f32, delta, rows: int) -> None:
+def residual_add(resid_f32, delta, rows: int, scale: float = 1.0) -> None:
+    """resid += scale * delta."""
     D = resid_f32.shape[-1]
     _need(resid_f32, "resid", torch.float32)
     _need(delta, "delta")
@@ -108,14 +110,17 @@ def residual_add(resid_f32, delta, rows: int) -> None:
         raise ValueError("residual_add: shape mismatch")
     L = _lib.load()
     _lib.check(L.he_residual_add(resid_f32.data_ptr(), delta.data_ptr(), rows * D,
-                                 dtype_code(delta.dtype), _stream()))
+                                 dtype_code(delta.dtype), float(scale), _stream()))
 
 
 @_op("silu_mul")
-def silu_mul(out, gate_up, rows: int, interleaved: bool = False, splits: int = 0) -> None:
+def silu_mul(out, gate_up, rows: int, interleaved: bool = False, splits: int = 0, *,
+             alpha: float = 1.0, limit: float = 0.0, up_shift: float = 0.0) -> None:
     """out[rows, I] = silu(gate) * up. gate_up: [rows, 2I] in out's dtype, or with
     splits > 0 the fp32 K slices [splits, rows, 2I] of the product. Its columns are all
-    gates then all ups, or, interleaved, gate i in column 2i and its up in 2i + 1."""
+    gates then all ups, or, interleaved, gate i in column 2i and its up in 2i + 1.
+    With constants it is the gated activation g' * sigmoid(alpha * g') * (u' + up_shift),
+    g' = min(gate, limit), u' = clamp(up, -limit, limit) (limit 0: unbounded)."""
     I = out.shape[-1]
     _need(out, "out")
     _need(gate_up, "gate_up", torch.float32 if splits > 0 else out.dtype)
@@ -125,8 +130,40 @@ def silu_mul(out, gate_up, rows: int, interleaved: bool = False, splits: int = 0
     if splits > 0 and tuple(gate_up.shape) != (splits, rows, 2 * I):
         raise ValueError("silu_mul: split sums must be [splits, rows, 2*I]")
     L = _lib.load()
-    _lib.check(L.he_silu_mul(out.data_ptr(), gate_up.data_ptr(), rows, I, int(interleaved), splits,
-                             dtype_code(out.dtype), _stream()))
+    _lib.check(L.he_gated_act(out.data_ptr(), gate_up.data_ptr(), rows, I, int(interleaved), splits,
+                              dtype_code(out.dtype), float(alpha), float(limit), float(up_shift), _stream()))
+
+
+@_op("add_dyt")
+def add_dyt(resid_f32, delta, weight, bias, alpha, out, rows: int, delta_scale: float = 1.0) -> None:
+    """resid += delta_scale * delta (if given); out = tanh(alpha * resid) * weight + bias (if out given).
+    alpha: a tensor of one element on the device; weight, bias: [D]; the three share a dtype."""
+    D = resid_f32.shape[-1]
+    _need(resid_f32, "resid", torch.float32)
+    _need(weight, "weight", shape=(D,))
+    _need(bias, "bias", weight.dtype, (D,))
+    _need(alpha, "alpha", weight.dtype)
+    if alpha.numel() != 1:
+        raise ValueError("add_dyt: alpha is one number")
+    if resid_f32.numel() < rows * D:
+        raise ValueError("add_dyt: resid smaller than the row count")
+    act = None
+    if out is not None:
+        _need(out, "out")
+        if out.shape[-1] != D or out.numel() < rows * D:
+            raise ValueError(f"add_dyt: out does not match [rows, {D}]")
+        act = out.dtype
+    if delta is not None:
+        _need(delta, "delta")
+        if delta.shape[-1] != D or delta.numel() < rows * D:
+            raise ValueError(f"add_dyt: delta does not match [rows, {D}]")
+        if act is not None and delta.dtype != act:
+            raise TypeError("add_dyt: delta and out must share a dtype")
+        act = delta.dtype
+    L = _lib.load()
+    _lib.check(L.he_add_dyt(resid_f32.data_ptr(), _ptr(delta), float(delta_scale), weight.data_ptr(),
+                            bias.data_ptr(), alpha.data_ptr(), _ptr(out), rows, D,
+                            dtype_code(act or torch.float32), dtype_code(weight.dtype), _stream()))
 
 
 @_op("add_rmsnorm")
@@ -430,20 +467,28 @@ def splitk_reduce(out, partial, bias, M: int, splits: int) -> None:
 @_op("qkv_rope_cache")
 def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, positions, row_seq,
                    seq_slot, page_table, inv_freq, rotary_dim: int, rows: int, H: int, KVH: int,
-                   hd: int, write_kv: bool) -> None:
-    """qkv: [rows, q_cols (+ 2 kv_cols)] projected rows without bias; bias (optional) has the same
-    column layout. Rotated q goes to q_out [rows, H*hd]; k, v go into the pools at
-    (slot, position) when write_kv."""
+                   hd: int, write_kv: bool, *, key_dim: int = 0, value_dim: int = 0,
+                   interleaved: bool = False, mscale: float = 1.0) -> None:
+    """qkv: [rows, q_cols + kv_cols + v_cols (+ more)] projected rows without bias; bias (optional)
+    covers those columns. Rotated q goes to q_out [rows, H*hd]; k, v go into the pools at
+    (slot, position) when write_kv. hd is the head size of q_out and of the cache pages; key_dim and
+    value_dim (0: hd) are the head sizes of the q/k and of the v columns, at most hd (q_out is then
+    padded with zeros, the pages keep the zeros they were made with). interleaved: frequency i turns
+    the dims (2i, 2i + 1) instead of (i, i + rotary_dim / 2); mscale multiplies cos and sin."""
     _need(qkv, "qkv")
     _need(q_out, "q_out")
     if qkv.dtype != q_out.dtype:
         raise TypeError("qkv_rope_cache: qkv and q_out must share a dtype")
     width = qkv.shape[-1]
-    if q_cols != H * hd or (write_kv and (kv_cols != KVH * hd or width != q_cols + 2 * kv_cols)):
+    kd, vd = key_dim or hd, value_dim or hd
+    v_cols = KVH * vd
+    if kd > hd or vd > hd or rotary_dim > kd:
+        raise ValueError("qkv_rope_cache: the rows' head sizes exceed the pages'")
+    if q_cols != H * kd or (write_kv and (kv_cols != KVH * kd or width < q_cols + kv_cols + v_cols)):
         raise ValueError("qkv_rope_cache: column layout does not match the head sizes")
     if not write_kv and width < q_cols:
         raise ValueError("qkv_rope_cache: qkv narrower than the query columns")
-    if qkv.numel() < rows * width or q_out.numel() < rows * q_cols:
+    if qkv.numel() < rows * width or q_out.numel() < rows * H * hd:
         raise ValueError("qkv_rope_cache: buffers smaller than the row count")
     _need(positions, "positions", torch.int32)
     _need(row_seq, "row_seq", torch.int32)
@@ -465,7 +510,9 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
     qb = kb = vb = None
     bias_code = F32
     if bias is not None:
-        _need(bias, "bias", shape=(width,))
+        _need(bias, "bias")
+        if bias.numel() < (q_cols + kv_cols + v_cols if write_kv else q_cols):
+            raise ValueError("qkv_rope_cache: bias shorter than the columns")
         bias_code = dtype_code(bias.dtype)
         bes = bias.element_size()
         qb = bias.data_ptr()
@@ -480,7 +527,7 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
         base, k_in, v_in, width, qb, kb, vb, bias_code, positions.data_ptr(), row_seq.data_ptr(),
         seq_slot.data_ptr(), _ptr(page_table) if write_kv else None, max_blocks, num_pages,
         _ptr(inv_freq) if rotary_dim else None, rotary_dim, rows, H, KVH if write_kv else 0, hd,
-        dtype_code(q_out.dtype), _stream()))
+        kd, vd, int(interleaved), float(mscale), dtype_code(q_out.dtype), _stream()))
 
 
 def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):
@@ -498,11 +545,18 @@ def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):
 @_op("attention_plain")
 def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,
                     H: int, KVH: int, hd: int, window: int, scale: float, most_keys: int = 0,
-                    workspace=None) -> None:
+                    workspace=None, *, chunk: int = 0, sinks=None, gate=None) -> None:
     """most_keys: a bound on the keys any sequence holds after the step, and workspace: fp32, of
     attention_plain_workspace_floats elements or more: the pages of a query then run in parallel
-    (a step of few queries over many keys); the result is the same bit for bit without them."""
+    (a step of few queries over many keys); the result is the same bit for bit without them.
+    chunk > 0: a query sees the keys of its own chunk of so many positions only (counted from
+    position 0). sinks [H]: a number a head that joins the softmax's denominator as exp(sink).
+    gate: a view [rows, H] of q's dtype (unit stride along heads, any row stride): the head's output
+    is multiplied by sigmoid(gate)."""
     _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd)
+    gate_ptr, gate_stride = _gate_view(gate, q, rows, H)
+    if sinks is not None:
+        _need(sinks, "sinks", shape=(H,))
     if workspace is not None:
         _need(workspace, "workspace", torch.float32)
     for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
@@ -513,12 +567,25 @@ def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_tab
     _lib.check(L.he_attention_plain(
         out.data_ptr(), q.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), positions.data_ptr(),
         row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(), page_table.shape[1],
-        kpool.shape[0], rows, H, KVH, hd, window, float(scale), dtype_code(q.dtype), int(most_keys),
+        kpool.shape[0], rows, H, KVH, hd, window, int(chunk), float(scale), _ptr(sinks),
+        dtype_code(sinks.dtype) if sinks is not None else F32, gate_ptr, gate_stride,
+        dtype_code(q.dtype), int(most_keys),
         _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream()))
 
 
-def attention_plain_workspace_floats(rows: int, H: int, hd: int, most_keys: int, window: int) -> int:
-    return int(_lib.load().he_attention_plain_workspace_floats(rows, H, hd, most_keys, window))
+def _gate_view(gate, q, rows: int, H: int):
+    """(pointer, row stride in elements) of a gate view [rows or more, H], or (None, 0)."""
+    if gate is None:
+        return None, 0
+    if not gate.is_cuda or gate.dtype != q.dtype or gate.dim() != 2 or gate.shape[1] != H \
+            or gate.shape[0] < rows or gate.stride(1) != 1:
+        raise ValueError(f"attention: gate must be a view [rows, {H}] of {q.dtype} with unit stride along heads")
+    return gate.data_ptr(), gate.stride(0)
+
+
+def attention_plain_workspace_floats(rows: int, H: int, hd: int, most_keys: int, window: int,
+                                     chunk: int = 0) -> int:
+    return int(_lib.load().he_attention_plain_workspace_floats(rows, H, hd, most_keys, window, chunk))
 
 
 def attention_decode_workspace_floats(rows: int, H: int, KVH: int, hd: int, max_keys: int) -> int:

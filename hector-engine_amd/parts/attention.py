@@ -8,6 +8,20 @@ before attention so that a query sees its own key (:1318-1326); the query at
 position p attends the keys (p - window, p], all of [0, p] without a window
 (kernels/attention.cu:60, :196, :696); kv head = h // (H / KVH) (:180);
 scale 1/sqrt(head_dim) (src/graph_builder.cpp:1328); then o = a Wo^T.
+
+Options of the same part, each off unless its parameter says otherwise:
+  value_dim   the values of a head are that wide (the keys stay head_dim wide). Keys, values and
+              the rotated q then live in heads of one padded size (the wider of the two, in steps
+              of 16 where the MFMA kernels run): the padding is zeros, the output matrix gets zero
+              columns for it, and every attention kernel sees one head size.
+  scale       the factor on q . k (default 1/sqrt(head_dim)).
+  chunk       position i sees j <= i only when floor(i / chunk) = floor(j / chunk); chunks are
+              counted from position 0 of the sequence.
+  sinks       a stored number per head joins the softmax's denominator as exp(sink_h); it has no
+              key and no value, is not scaled and counts once.
+  head_gate   head h's output is multiplied by sigmoid(g_h), g = Wg n with one row of Wg a head;
+              the rows of Wg ride behind q||k||v in the one product.
+  names       the suffixes of its tensors (q, k, v, o, q_bias, k_bias, v_bias, o_bias, sinks, gate).
 """
 from __future__ import annotations
 
@@ -18,7 +32,11 @@ import torch
 
 from ..kernels import kv_layout, ops, routes
 from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, StepContext, TensorSpec,
-                   build_part, param, register_part)
+                   build_part, param, register_part, tensor_name)
+
+_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+          "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
+          "sinks": "sinks", "gate": "gate.weight"}
 from .linear import Linear
 
 
@@ -56,8 +74,22 @@ class Attention(Mixer):
         self.window = param(params, "window", int, 0)
         self.kv_projection = param(params, "kv_projection", bool, True)
         self.scale = param(params, "scale", float, 1.0 / math.sqrt(self.hd))
+        self.vd = param(params, "value_dim", int, self.hd)
+        self.chunk = param(params, "chunk", int, 0)
+        self.has_sinks = param(params, "sinks", bool, False)
+        self.head_gate = param(params, "head_gate", bool, False)
+        names = param(params, "names", dict, {})
+        self._names = {k: tensor_name(prefix, names, k, d) for k, d in _NAMES.items()}
         if self.H % self.KVH:
             raise ValueError(f"attention: {self.H} heads are not a multiple of {self.KVH} kv heads")
+        if self.vd <= 0 or self.chunk < 0:
+            raise ValueError(f"attention: value_dim {self.vd} must be positive, chunk {self.chunk} not negative")
+        # the one head size of the cache pages, of the rotated q and of the attention's output
+        self.pd = max(self.hd, self.vd)
+        mfma = env.dtype == torch.bfloat16 and getattr(env, "fast_kernels", True)
+        if mfma and (self.hd != self.vd or self.pd % 16) and self.pd <= 256:
+            self.pd = (self.pd + 15) // 16 * 16
+        self.sinks: torch.Tensor | None = None
         self.position = build_part("position", param(params, "position", PartSpec, PartSpec("none")),
                                    prefix, env)
         self.qkv: Linear | None = None
@@ -65,52 +97,72 @@ class Attention(Mixer):
         self.o_proj: Linear | None = None
         self._chosen: dict[tuple, routes.Route] = {}      # (all one-token, dtype) -> route, for one version of the table
         self._chosen_version = -1
-        self.fast = env.dtype == torch.bfloat16 and getattr(env, "fast_kernels", True) \
-            and self.hd % 16 == 0 and self.hd <= 256 and self.scale > 0   # else the plain kernel
+        self.fast = mfma and self.pd % 16 == 0 and self.pd <= 256 and self.scale > 0   # else the plain kernel
+        # what the fused one-token kernel and the kernels without these options do not take
+        self.extras = self.chunk > 0 or self.has_sinks or self.head_gate
 
     def children(self):
         return [self.position]
 
     def kv_need(self):
         # pages in the order the attention kernels read their operands
-        return KVNeed(self.KVH, self.hd, self.window, k_page_elems=kv_layout.k_page_elems(self.hd),
-                      v_page_elems=kv_layout.v_page_elems(self.hd))
+        return KVNeed(self.KVH, self.pd, self.window, k_page_elems=kv_layout.k_page_elems(self.pd),
+                      v_page_elems=kv_layout.v_page_elems(self.pd))
 
     def tensor_specs(self):
-        p, hd = self.prefix, self.hd
-        specs = {p + "q_proj.weight": TensorSpec((self.H * hd, self.hidden)),
-                 p + "o_proj.weight": TensorSpec((self.hidden, self.H * hd))}
+        n, hd, vd = self._names, self.hd, self.vd
+        specs = {n["q"]: TensorSpec((self.H * hd, self.hidden)),
+                 n["o"]: TensorSpec((self.hidden, self.H * vd))}
         if self.kv_projection:
-            specs[p + "k_proj.weight"] = TensorSpec((self.KVH * hd, self.hidden))
-            specs[p + "v_proj.weight"] = TensorSpec((self.KVH * hd, self.hidden))
+            specs[n["k"]] = TensorSpec((self.KVH * hd, self.hidden))
+            specs[n["v"]] = TensorSpec((self.KVH * vd, self.hidden))
         if self.qkv_bias:
-            specs[p + "q_proj.bias"] = TensorSpec((self.H * hd,))
+            specs[n["q_bias"]] = TensorSpec((self.H * hd,))
             if self.kv_projection:
-                specs[p + "k_proj.bias"] = TensorSpec((self.KVH * hd,))
-                specs[p + "v_proj.bias"] = TensorSpec((self.KVH * hd,))
+                specs[n["k_bias"]] = TensorSpec((self.KVH * hd,))
+                specs[n["v_bias"]] = TensorSpec((self.KVH * vd,))
         if self.out_bias:
-            specs[p + "o_proj.bias"] = TensorSpec((self.hidden,))
+            specs[n["o_bias"]] = TensorSpec((self.hidden,))
+        if self.has_sinks:
+            specs[n["sinks"]] = TensorSpec((self.H,), ("normal", 1.0))
+        if self.head_gate:
+            specs[n["gate"]] = TensorSpec((self.H, self.hidden))
         specs.update(self.position.tensor_specs())
         return specs
 
     def bind(self, tensors):
-        p = self.prefix
-        names = ["q_proj"] + (["k_proj", "v_proj"] if self.kv_projection else [])
-        ws = [tensors.pop(p + n + ".weight") for n in names]
+        p, n = self.prefix, self._names
+        names = ["q"] + (["k", "v"] if self.kv_projection else [])
+        ws = [tensors.pop(n[x]) for x in names]
+        gate_w = tensors.pop(n["gate"]) if self.head_gate else None
+        if gate_w is not None:
+            ws.append(gate_w)          # the gate's rows ride behind q||k||v: one product
         if len({w.dtype for w in ws}) != 1:
             raise TypeError(f"{p}q/k/v projections are stored in different dtypes")
         w = torch.cat(ws, 0).contiguous() if len(ws) > 1 else ws[0]
         b = None
         if self.qkv_bias:
-            bs = [tensors.pop(p + n + ".bias") for n in names]
+            bs = [tensors.pop(n[x + "_bias"]) for x in names]
             if len({x.dtype for x in bs}) != 1:
                 raise TypeError(f"{p}q/k/v biases are stored in different dtypes")
             b = torch.cat(bs, 0).contiguous() if len(bs) > 1 else bs[0]
-        del ws
         self.qkv = Linear(w, b)
         q_rows = self.H * self.hd
-        self.q_only = Linear(w[:q_rows], None if b is None else b[:q_rows])
-        self.o_proj = Linear(tensors[p + "o_proj.weight"], tensors.get(p + "o_proj.bias"))
+        if gate_w is not None and self.kv_projection:
+            self.q_only = Linear(torch.cat([ws[0], gate_w], 0).contiguous(), None if b is None else b[:q_rows])
+        else:
+            self.q_only = Linear(w[:q_rows + (self.H if gate_w is not None else 0)],
+                                 None if b is None else b[:q_rows])
+        del ws
+        wo = tensors[n["o"]]
+        if self.pd != self.vd:
+            # zero columns where the attention's output holds the padding of a head
+            padded = torch.zeros((self.hidden, self.H, self.pd), dtype=wo.dtype, device=wo.device)
+            padded[:, :, :self.vd] = wo.view(self.hidden, self.H, self.vd)
+            wo = padded.view(self.hidden, self.H * self.pd)
+        self.o_proj = Linear(wo, tensors.get(n["o_bias"]))
+        if self.has_sinks:
+            self.sinks = tensors[n["sinks"]]
         self.position.bind(tensors)
 
     def forward(self, x, ctx: StepContext, cache: LayerCache):
@@ -124,8 +176,10 @@ class Attention(Mixer):
         if route is None:
             rot = self.position.rotary()
             case = AttentionCase(
-                all_single=ctx.all_single, fast=self.fast,
-                fusable=not self.position.custom and rot is not None
+                all_single=ctx.all_single, fast=self.fast and not self.extras,
+                fusable=not self.position.custom and rot is not None and not self.extras
+                and self.hd == self.vd == self.pd
+                and not self.position.interleaved and self.position.mscale == 1.0
                 and ops.attention_decode_fused_ok(self.H, self.KVH, self.hd, rot[1]))
             route = self._chosen[key] = routes.choose("attention", (ctx.env.dtype,), case)
         return route.run(self, x, ctx, cache)
@@ -157,7 +211,8 @@ class Attention(Mixer):
         return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, sink=ctx.take_sink())
 
     def _encoded_q(self, x, ctx: StepContext, cache: LayerCache):
-        """q with bias and position encoding, after the new keys and values went into the cache."""
+        """(q with bias and position encoding, after the new keys and values went into the cache;
+        the heads' gates as a view of the projection's rows, or None)."""
         rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
         writes = cache.writes
         proj = self.qkv if writes else self.q_only
@@ -171,29 +226,35 @@ class Attention(Mixer):
             qv = qkv[:, :q_cols].unflatten(1, (H, hd))
             kv = qkv[:, q_cols:q_cols + kv_cols].unflatten(1, (KVH, hd)) if writes else None
             self.position.apply(qv, kv, ctx)
-        q = ctx.alloc((rows, H * hd))
+        q = ctx.alloc((rows, H * self.pd))
         inv_freq, r = rot if rot is not None else (None, 0)
         ops.qkv_rope_cache(q, cache.kpool, cache.vpool, qkv, H * hd, KVH * hd,
                            proj.bias if fused_bias else None, ctx.positions, ctx.row_seq,
-                           ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, hd, writes)
-        return q
+                           ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, self.pd, writes,
+                           key_dim=hd, value_dim=self.vd, interleaved=self.position.interleaved,
+                           mscale=self.position.mscale)
+        gate = None
+        if self.head_gate:
+            at = H * hd + (KVH * (hd + self.vd) if writes else 0)
+            gate = qkv[:rows, at:at + H]
+        return q, gate
 
     def _run_plain(self, x, ctx: StepContext, cache: LayerCache):
         """The plain kernel: one fixed order per (query, head), in the precision of the cache."""
-        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
-        q = self._encoded_q(x, ctx, cache)
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.pd
+        q, gate = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
-        floats = ops.attention_plain_workspace_floats(rows, H, hd, ctx.most_keys, self.window)
+        floats = ops.attention_plain_workspace_floats(rows, H, hd, ctx.most_keys, self.window, self.chunk)
         ws = ctx.alloc((floats,), torch.float32) if floats else None
         ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                             ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                            self.scale, ctx.most_keys, ws)
+                            self.scale, ctx.most_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate)
         return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
 
     def _run_mfma_one_token(self, x, ctx: StepContext, cache: LayerCache):
         """One-token steps of the head sizes and encodings the fused kernel does not take."""
-        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
-        q = self._encoded_q(x, ctx, cache)
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.pd
+        q, _ = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
         floats = ops.attention_decode_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
         ws = ctx.alloc((max(floats, 1),), torch.float32)
@@ -204,8 +265,8 @@ class Attention(Mixer):
 
     def _run_mfma_prompt(self, x, ctx: StepContext, cache: LayerCache):
         """Prompt steps and mixed steps."""
-        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
-        q = self._encoded_q(x, ctx, cache)
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.pd
+        q, _ = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
         # few queries against many keys (a continuation of a long sequence): the keys in parts
         most = ctx.most_keys

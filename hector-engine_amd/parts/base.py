@@ -51,10 +51,13 @@ class LayerSpec:
 @dataclasses.dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a layer. cache_from names an earlier entry of the schedule
-    whose cache this run reads instead of writing one of its own."""
+    whose cache this run reads instead of writing one of its own. add_embedding: the embedding's
+    output (the stream as it was before the first run) is added to the stream right before this
+    run (a pass over a stretch of layers that starts again from the input)."""
 
     layer: int
     cache_from: int | None = None
+    add_embedding: bool = False
 
 
 @dataclasses.dataclass
@@ -218,9 +221,10 @@ class Norm(Part):
         return None
 
     def add_norm(self, resid: torch.Tensor, delta, rows: int, ctx: StepContext,
-                 want_out: bool = True) -> torch.Tensor | None:
-        """resid (fp32 [rows, D], in place) += delta (a tensor in the activation dtype, or
-        None); returns norm(resid) in the activation dtype (or None when want_out is False)."""
+                 want_out: bool = True, delta_scale: float = 1.0) -> torch.Tensor | None:
+        """resid (fp32 [rows, D], in place) += delta_scale * delta (a tensor in the activation
+        dtype, or None); returns norm(resid) in the activation dtype (or None when want_out is
+        False)."""
         raise NotImplementedError
 
 
@@ -228,6 +232,10 @@ class PositionEncoding(Part):
     # True for an encoding that must run through apply() on q and k; False for a
     # rotation the fused q/k kernel applies (rotary() gives its table) or for none.
     custom = False
+    # how a rotation that rotary() describes pairs its dims and scales its cos and sin: frequency
+    # i turns (i, i + r/2), or, interleaved, (2i, 2i + 1); mscale multiplies cos and sin
+    interleaved = False
+    mscale = 1.0
 
     def rotary(self) -> tuple[torch.Tensor, int] | None:
         """(inv_freq fp32 [r/2], r) when the encoding is a rotation the fused
@@ -335,17 +343,19 @@ class ResidualStream:
         self.resid = resid
         self.rows = rows
         self.pending: torch.Tensor | None = None
+        self.pending_scale = 1.0                               # the stream gains pending_scale * pending
         self.prepared: tuple[Norm, NormedRows] | None = None   # rows already made for that norm
 
-    def add(self, delta, ctx: StepContext) -> None:
-        """delta: a tensor [rows, D], or None when the producer has added its result through a
-        ResidualSink."""
+    def add(self, delta, ctx: StepContext, scale: float = 1.0) -> None:
+        """The stream gains scale * delta. delta: a tensor [rows, D], or None when the producer
+        has added its result through a ResidualSink."""
         if delta is None:
             return
         self.prepared = None
         if self.pending is not None:
             self.materialize(ctx)
         self.pending = delta
+        self.pending_scale = scale
 
     def sink_for(self, norm: Norm | None, ctx: StepContext) -> "ResidualSink | None":
         """A sink for the part that runs next, when `norm` (the norm that will read the stream
@@ -362,14 +372,17 @@ class ResidualStream:
         prepared, self.prepared = self.prepared, None
         if prepared is not None and prepared[0] is norm and self.pending is None:
             return prepared[1] if rows_ok else prepared[1].tensor(ctx)
-        out = norm.add_norm(self.resid, self.pending, self.rows, ctx)
+        if self.pending is not None and self.pending_scale != 1.0:
+            out = norm.add_norm(self.resid, self.pending, self.rows, ctx, delta_scale=self.pending_scale)
+        else:
+            out = norm.add_norm(self.resid, self.pending, self.rows, ctx)
         self.pending = None
         return out
 
     def materialize(self, ctx: StepContext) -> torch.Tensor:
         if self.pending is not None:
             from ..kernels import ops
-            ops.residual_add(self.resid, self.pending, self.rows)
+            ops.residual_add(self.resid, self.pending, self.rows, self.pending_scale)
             self.pending = None
         return self.resid
 
@@ -402,6 +415,15 @@ def build_part(category: str, spec: PartSpec, prefix: str, env: BuildEnv) -> Par
         raise KeyError(f"no {category} of kind '{spec.kind}' is registered; "
                        f"registered: {sorted(_registries.get(category, {}))}") from None
     return factory(dict(spec.params), prefix, env)
+
+
+def tensor_name(prefix: str, names: dict | None, key: str, default: str) -> str:
+    """The full name of a part's tensor `key`: the part's prefix followed by the suffix that
+    `names` (a part's optional `names` parameter) gives for the key, else by `default`. An empty
+    suffix stands for the prefix itself without its trailing dot: a vector stored under the very
+    name its companions hang their own suffixes on ('x.norm' beside 'x.norm.b')."""
+    suffix = default if not names or key not in names else names[key]
+    return prefix + suffix if suffix else prefix.rstrip(".")
 
 
 def registered(category: str) -> list[str]:

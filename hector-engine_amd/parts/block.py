@@ -3,7 +3,10 @@
 (reference: src/graph_builder.cpp:1195, :1366-1374, :1396, :1443). Each
 residual add is carried as pending and fused into the next norm, or, with few
 rows, done by the last product of the mixer / feed-forward, which then also prepares
-the rows of the norm that follows (parts.base.ResidualSink)."""
+the rows of the norm that follows (parts.base.ResidualSink).
+
+residual_scale m (1 unless given): x = x + m * mixer(norm1(x)); x = x + m * feed_forward(norm2(x)).
+A layer without a feed-forward (feed_forward None) is the first line alone."""
 from __future__ import annotations
 
 from .base import (Block, BuildEnv, LayerCache, PartSpec, ResidualStream, StepContext,
@@ -19,13 +22,16 @@ class PreNormBlock(Block):
                                      prefix + names["mixer_norm"] + ".", env)
         self.mixer = build_part("mixer", param(params, "mixer", PartSpec),
                                 prefix + names["mixer"] + ".", env)
-        self.ff_norm = build_part("norm", param(params, "feed_forward_norm", PartSpec),
-                                  prefix + names["feed_forward_norm"] + ".", env)
-        self.feed_forward = build_part("feed_forward", param(params, "feed_forward", PartSpec),
-                                       prefix + names["feed_forward"] + ".", env)
+        self.residual_scale = param(params, "residual_scale", float, 1.0)
+        self.ff_norm = self.feed_forward = None
+        if param(params, "feed_forward", PartSpec, None) is not None:
+            self.ff_norm = build_part("norm", param(params, "feed_forward_norm", PartSpec),
+                                      prefix + names["feed_forward_norm"] + ".", env)
+            self.feed_forward = build_part("feed_forward", param(params, "feed_forward", PartSpec),
+                                           prefix + names["feed_forward"] + ".", env)
 
     def children(self):
-        return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
+        return [p for p in (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward) if p is not None]
 
     def first_norm(self):
         return self.mixer_norm
@@ -42,13 +48,17 @@ class PreNormBlock(Block):
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
         after = ctx.next_norm                  # reads the stream once this block is done
+        m = self.residual_scale
+        sinks = m == 1.0                       # a product that adds into the stream itself adds unscaled
         n = stream.normed(self.mixer_norm, ctx, self.mixer.accepts_normed_rows)
-        ctx.sink = stream.sink_for(self.ff_norm, ctx)
+        ctx.sink = stream.sink_for(self.ff_norm if self.feed_forward is not None else after, ctx) if sinks else None
         delta = self.mixer.forward(n, ctx, cache)
         ctx.sink = None
-        stream.add(delta, ctx)
+        stream.add(delta, ctx, m)
+        if self.feed_forward is None:
+            return
         n = stream.normed(self.ff_norm, ctx, self.feed_forward.accepts_normed_rows)
-        ctx.sink = stream.sink_for(after, ctx)
+        ctx.sink = stream.sink_for(after, ctx) if sinks else None
         delta = self.feed_forward.forward(n, ctx)
         ctx.sink = None
-        stream.add(delta, ctx)
+        stream.add(delta, ctx, m)

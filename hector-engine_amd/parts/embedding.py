@@ -11,7 +11,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import BuildEnv, Part, StepContext, TensorSpec, param, register_part
+from .base import BuildEnv, Part, StepContext, TensorSpec, param, register_part, tensor_name
 from .linear import Linear
 
 
@@ -21,17 +21,19 @@ class TokenEmbedding(Part):
         super().__init__(prefix, env)
         self.vocab = param(params, "vocab_size", int)
         self.hidden = param(params, "hidden_size", int)
+        self.scale = param(params, "scale", float, 1.0)      # h[t] = E[id_t] * scale
+        self._name = tensor_name(prefix, param(params, "names", dict, {}), "weight", "weight")
         self.table: torch.Tensor | None = None
 
     def tensor_specs(self):
-        return {self.prefix + "weight": TensorSpec((self.vocab, self.hidden))}
+        return {self._name: TensorSpec((self.vocab, self.hidden))}
 
     def bind(self, tensors):
-        self.table = tensors[self.prefix + "weight"]
+        self.table = tensors[self._name]
 
     def forward(self, ids: torch.Tensor, rows: int, ctx: StepContext) -> torch.Tensor:
         out = ctx.alloc((rows, self.hidden), torch.float32)
-        ops.embedding(out, self.table, ids, rows)
+        ops.embedding(out, self.table, ids, rows, self.scale)
         return out
 
 
@@ -44,15 +46,16 @@ class LinearHead(Part):
         self.vocab = param(params, "vocab_size", int)
         self.hidden = param(params, "hidden_size", int)
         self.tied_to = param(params, "tied_to", str, "")   # full name of the tensor it shares
+        self._name = tensor_name(prefix, param(params, "names", dict, {}), "weight", "weight")
         self.linear: Linear | None = None
 
     def tensor_specs(self):
         if self.tied_to:
             return {}
-        return {self.prefix + "weight": TensorSpec((self.vocab, self.hidden))}
+        return {self._name: TensorSpec((self.vocab, self.hidden))}
 
     def bind(self, tensors):
-        name = self.tied_to or self.prefix + "weight"
+        name = self.tied_to or self._name
         self.linear = Linear(tensors[name])
 
     def forward(self, x: torch.Tensor, rows: int, ctx: StepContext) -> torch.Tensor:

@@ -2,13 +2,19 @@
 no biases (reference: src/graph_builder.cpp:1415-1428,
 kernels/activations.cu:183-198). Gate and up are one product over the
 row-concatenated weight gate||up (the reference's optional fusion:
-src/graph_builder.cpp:1400-1414)."""
+src/graph_builder.cpp:1400-1414).
+
+activation "clamped_swiglu" is the same feed-forward through a bounded gate:
+g' = min(g, limit), u' = clamp(u, -limit, limit), act = g' * sigmoid(alpha * g') * (u' + 1), with
+the parameters `limit` and `alpha` (1.702 unless given). names: the suffixes of its tensors
+(gate, up, down)."""
 from __future__ import annotations
 
 import torch
 
 from ..kernels import ops
-from .base import BuildEnv, FeedForward, NormedRows, PieceRows, StepContext, TensorSpec, param, register_part
+from .base import (BuildEnv, FeedForward, NormedRows, PieceRows, StepContext, TensorSpec, param, register_part,
+                   tensor_name)
 from .linear import Linear
 
 # rows of the intermediate activations held at once in a long prompt step
@@ -24,22 +30,32 @@ class GatedMLP(FeedForward):
         self.hidden = param(params, "hidden_size", int)
         self.inter = param(params, "intermediate_size", int)
         act = param(params, "activation", str, "silu")
-        if act not in ("silu", "swish"):
+        if act in ("silu", "swish"):
+            self.act = {}                         # SiLU(gate) * up
+        elif act == "clamped_swiglu":
+            limit = param(params, "limit", float)
+            if limit <= 0:
+                raise ValueError(f"gated_mlp: limit {limit} must be positive")
+            self.act = {"alpha": param(params, "alpha", float, 1.702), "limit": limit, "up_shift": 1.0}
+        else:
             raise ValueError(f"gated_mlp: unsupported activation '{act}'")
+        names = param(params, "names", dict, {})
+        self._names = {k: tensor_name(prefix, names, k, d) for k, d in
+                       (("gate", "gate_proj.weight"), ("up", "up_proj.weight"), ("down", "down_proj.weight"))}
         self.gate_up: Linear | None = None
         self.down: Linear | None = None
 
     def tensor_specs(self):
-        p = self.prefix
+        n = self._names
         return {
-            p + "gate_proj.weight": TensorSpec((self.inter, self.hidden)),
-            p + "up_proj.weight": TensorSpec((self.inter, self.hidden)),
-            p + "down_proj.weight": TensorSpec((self.hidden, self.inter)),
+            n["gate"]: TensorSpec((self.inter, self.hidden)),
+            n["up"]: TensorSpec((self.inter, self.hidden)),
+            n["down"]: TensorSpec((self.hidden, self.inter)),
         }
 
     def bind(self, tensors):
-        p = self.prefix
-        g, u = tensors.pop(p + "gate_proj.weight"), tensors.pop(p + "up_proj.weight")
+        p, n = self.prefix, self._names
+        g, u = tensors.pop(n["gate"]), tensors.pop(n["up"])
         if g.dtype != u.dtype:
             raise TypeError(f"{p}gate_proj and up_proj are stored in different dtypes")
         # gate and up rows alternate (gate i at row 2i, its up at 2i + 1): the four neighbouring
@@ -48,13 +64,13 @@ class GatedMLP(FeedForward):
         w = torch.stack([g, u], 1).reshape(2 * g.shape[0], g.shape[1])
         self.gate_up = Linear(w.contiguous())
         del g, u, w
-        self.down = Linear(tensors[p + "down_proj.weight"])
+        self.down = Linear(tensors[n["down"]])
 
     def forward(self, x, ctx: StepContext):
         rows = ctx.rows
         if rows <= _ROW_CHUNK:
             act = x.scaled.dtype if isinstance(x, NormedRows) else x.dtype
-            if self.gate_up.gated_silu_rows(rows, ctx, act):
+            if not self.act and self.gate_up.gated_silu_rows(rows, ctx, act):
                 # up to 64 rows: the activation is the product's epilogue, and its result goes to the
                 # down projection piece-major where that reads it so
                 pieces = self.inter % 8 == 0 and self.down.reads_pieces(rows, ctx) and self.gate_up.gated_pieces(rows)
@@ -63,7 +79,7 @@ class GatedMLP(FeedForward):
                 return self.down(PieceRows(h) if pieces else h, rows, ctx, sink=ctx.take_sink())
             h = ctx.alloc((rows, self.inter))
             gu = self.gate_up(x, rows, ctx)
-            ops.silu_mul(h, gu, rows, True)
+            ops.silu_mul(h, gu, rows, True, **self.act)
             return self.down(h, rows, ctx, sink=ctx.take_sink())
         if not isinstance(x, torch.Tensor):
             x = x.tensor(ctx)
@@ -73,7 +89,7 @@ class GatedMLP(FeedForward):
             turn = ctx.scratch.mark()
             h = ctx.alloc((n, self.inter))
             gu = self.gate_up(x[r0:r0 + n], n, ctx)
-            ops.silu_mul(h, gu, n, True)
+            ops.silu_mul(h, gu, n, True, **self.act)
             self.down(h, n, ctx, out=out[r0:r0 + n])
             ctx.scratch.release(turn)       # the next turn reuses h and gate||up
         return out

@@ -7,7 +7,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import BuildEnv, Norm, StepContext, TensorSpec, param, register_part
+from .base import BuildEnv, Norm, StepContext, TensorSpec, param, register_part, tensor_name
 
 
 @register_part("norm", "rmsnorm")
@@ -27,7 +27,42 @@ class RMSNorm(Norm):
     def carried(self):
         return self.weight, self.eps
 
-    def add_norm(self, resid, delta, rows, ctx: StepContext, want_out: bool = True):
+    def add_norm(self, resid, delta, rows, ctx: StepContext, want_out: bool = True, delta_scale: float = 1.0):
         out = ctx.alloc((rows, self.size)) if want_out else None
+        if delta is not None and delta_scale != 1.0:
+            ops.residual_add(resid, delta, rows, delta_scale)
+            delta = None
         ops.add_rmsnorm(resid, delta, self.weight, out, rows, self.eps)
+        return out
+
+
+@register_part("norm", "dynamic_tanh")
+class DynamicTanh(Norm):
+    """y = tanh(alpha * x) * weight + bias with a stored scalar alpha and vectors weight, bias: it
+    stands where a norm would and computes neither a mean nor a variance, so no row is reduced and no
+    pair of products can carry it. Computed in fp32 on the fp32 residual stream, fused with the
+    pending (scaled) residual add. names: suffixes of its tensors (weight, bias, alpha)."""
+
+    def __init__(self, params: dict, prefix: str, env: BuildEnv):
+        super().__init__(prefix, env)
+        self.size = param(params, "size", int)
+        names = param(params, "names", dict, {})
+        self._names = {k: tensor_name(prefix, names, k, k) for k in ("weight", "bias", "alpha")}
+        self.weight = self.bias = self.alpha = None
+
+    def tensor_specs(self):
+        n = self._names
+        return {n["weight"]: TensorSpec((self.size,), ("gain", 1.0, 0.1)),
+                n["bias"]: TensorSpec((self.size,), ("normal", 0.02)),
+                n["alpha"]: TensorSpec((), ("gain", 0.5, 0.05))}
+
+    def bind(self, tensors):
+        n = self._names
+        self.weight, self.bias, self.alpha = tensors[n["weight"]], tensors[n["bias"]], tensors[n["alpha"]]
+        if not (self.weight.dtype == self.bias.dtype == self.alpha.dtype):
+            raise TypeError(f"{self.prefix}: weight, bias and alpha are stored in different dtypes")
+
+    def add_norm(self, resid, delta, rows, ctx: StepContext, want_out: bool = True, delta_scale: float = 1.0):
+        out = ctx.alloc((rows, self.size)) if want_out else None
+        ops.add_dyt(resid, delta, self.weight, self.bias, self.alpha, out, rows, delta_scale)
         return out
