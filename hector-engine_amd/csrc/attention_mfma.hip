@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ page_table, int max_blocks,
-    int num_pages, int H, int KVH, int window, float scale) {
+    int num_pages, int H, int KVH, int window, float scale, AttnExtras ex) {
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const bool q_ok = qi < q_len;
   const int pos = start + qi;             // its absolute position
   const int hi = q_ok ? pos : -1;
-  const int lo = (window > 0 && q_ok) ? max(0, pos + 1 - window) : 0;
+  const int lo = q_ok ? attn_first(pos, window, ex.chunk) : 0;
   bf16x8 qf[KS];
   load_q<NT>(qf, q + ((int64_t)(row0 + max(0, min(qi, q_len - 1))) * H + h) * HD, q_ok, lg);
 
@@ -68,11 +68,11 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 
   const int last_pos = start + min(q0 + 15, q_len - 1);
   const int first_pos = start + q0;
-  const int tile_lo = window > 0 ? max(0, first_pos + 1 - window) : 0;
+  const int tile_lo = attn_first(first_pos, window, ex.chunk);
   // every query of a full tile sees the keys from the last query's window start to the
   // first query's position
   const bool full_tile = q0 + 15 < q_len;
-  const int clear_lo = window > 0 ? max(0, last_pos + 1 - window) : 0;
+  const int clear_lo = attn_first(last_pos, window, ex.chunk);
   const int clear_hi = full_tile ? first_pos : -1;
   attend_range<NT, true>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, tile_lo & ~31,
                    (last_pos & ~31) + 32, lo, hi, clear_lo, clear_hi, scale * 1.4426950408889634f,
@@ -80,7 +80,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   float l = st.l;
   l = xor32_sum(xor16_sum(l));
   if (!q_ok) return;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  l += attn_sink_term(ex, h, st.m);
+  const float inv = (l > 0.f ? 1.f / l : 0.f) * attn_gate(ex, row0 + qi, h);
   uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD;
 #pragma unroll
   for (int dt = 0; dt < NT; ++dt) {
@@ -108,7 +109,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
-    int num_pages, int H, int KVH, int head_tiles, int window, float scale) {
+    int num_pages, int H, int KVH, int head_tiles, int window, float scale, AttnExtras ex) {
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
   const int lane = threadIdx.x;
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   }
   const int slot = seq_slot[seq];
   const int n_keys = positions[row] + 1;
-  const int first = window > 0 ? max(0, n_keys - window) : 0;
+  const int first = attn_first(n_keys - 1, window, ex.chunk);
   const int span_lo = first & ~31;
   int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
   chunk = max(DECODE_MIN_CHUNK, (chunk + 31) & ~31);
@@ -154,7 +155,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   l = xor32_sum(xor16_sum(l));
   if (nsplit == 1) {                      // nothing to merge
     if (!h_ok) return;
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    l += attn_sink_term(ex, h, st.m);
+    const float inv = (l > 0.f ? 1.f / l : 0.f) * attn_gate(ex, row, h);
 #pragma unroll
     for (int dt = 0; dt < NT; ++dt) {
       uint2 w;
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 __global__ __launch_bounds__(256) void attention_merge_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq, int H, int HD,
-    int nsplit, int window, int all_parts, int out_pieces) {
+    int nsplit, int window, int all_parts, int out_pieces, AttnExtras ex) {
   __shared__ float wgt[64];
   __shared__ float part[4][256];
   const int h = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -206,7 +208,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(
     active = 0;
     if (live) {
       const int n_keys = positions[row] + 1;
-      const int first = window > 0 ? max(0, n_keys - window) : 0;
+      const int first = attn_first(n_keys - 1, window, ex.chunk);
       const int span_lo = first & ~31;
       int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
       chunk = max(DECODE_MIN_CHUNK, (chunk + 31) & ~31);
@@ -230,10 +232,11 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(
   load_slices(ov, 0, 0);
   const float M = wave_max(m);
   const float w = m > -INFINITY ? __builtin_amdgcn_exp2f(m - M) : 0.f;   // m is in the base-2 domain
-  const float L = wave_sum(l * w);          // every wavefront computes the same weights
+  float L = wave_sum(l * w);                // every wavefront computes the same weights
   if (wave == 0) wgt[lane] = w;             // 0 from `active` on
   __syncthreads();
-  const float inv = L > 0.f ? 1.f / L : 0.f;
+  if (live) L += attn_sink_term(ex, h, M);
+  const float inv = (L > 0.f ? 1.f / L : 0.f) * (live ? attn_gate(ex, row, h) : 1.f);
   for (int d0 = 0; d0 < HD; d0 += 256) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int s0 = 0; s0 < active; s0 += 4 * MERGE_PER) {
@@ -301,7 +304,10 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
                                         const void* page_table, int max_blocks, int num_pages,
                                         int rows, int H, int KVH, int hd, int window, float scale,
                                         int max_keys, void* workspace_f32,
-                                        int64_t workspace_floats, void* stream) {
+                                        int64_t workspace_floats, int chunk, const void* sinks,
+                                        int sinks_dtype, const void* gate, int64_t gate_stride,
+                                        void* stream) {
+  const AttnExtras ex = {sinks, sinks_dtype, (const uint16_t*)gate, gate_stride, chunk};
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0 && max_keys > 0,
              "he_attention_decode_bf16: bad sizes");
   HE_REQUIRE(scale > 0.f, "he_attention_decode_bf16: the score scale must be positive");
@@ -331,12 +337,12 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
                            (const uint16_t*)kpool, (const uint16_t*)vpool,
                            (const int32_t*)positions, (const int32_t*)row_seq,
                            (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,
-                           num_pages, H, KVH, head_tiles, window, scale)));
+                           num_pages, H, KVH, head_tiles, window, scale, ex)));
   int rc = he_check_launch("he_attention_decode_bf16");
   if (rc || nsplit == 1) return rc;
   attention_merge_kernel<<<dim3(H, rows), 256, 0, s>>>(
       (uint16_t*)out, ws_o, ws_ml, (const int32_t*)positions, (const int32_t*)row_seq, H, hd,
-      nsplit, window, 0, 0);
+      nsplit, window, 0, 0, ex);
   return he_check_launch("he_attention_decode_bf16 merge");
 }
 
@@ -345,7 +351,7 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
 // Parts are added in their order. Every part was stored; out is row-major.
 __global__ __launch_bounds__(256) void attention_merge_rows_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
-    int64_t pairs, int HD, int nsplit) {
+    int64_t pairs, int HD, int nsplit, int H, AttnExtras ex) {
   const int lane = threadIdx.x & 63;
   const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);   // row * H + h
   if (pair >= pairs) return;
@@ -363,8 +369,9 @@ __global__ __launch_bounds__(256) void attention_merge_rows_kernel(
   // lane s has the weight of part s (0 from nsplit on); all lanes take part in the sums
   const float M = wave_max(ml.x);
   const float w = ml.x > -INFINITY ? __builtin_amdgcn_exp2f(ml.x - M) : 0.f;   // base-2 domain
-  const float L = wave_sum(ml.y * w);
-  const float inv = L > 0.f ? 1.f / L : 0.f;
+  const int h = (int)(pair % H);
+  const float L = wave_sum(ml.y * w) + attn_sink_term(ex, h, M);
+  const float inv = (L > 0.f ? 1.f / L : 0.f) * attn_gate(ex, pair / H, h);
   for (int d0 = 2 * lane; d0 < HD; d0 += 128) {
     float2 acc = make_float2(0.f, 0.f);
     for (int s0 = 0; s0 < nsplit; s0 += MERGE_PER) {
@@ -382,13 +389,13 @@ __global__ __launch_bounds__(256) void attention_merge_rows_kernel(
 }
 
 int he_attention_merge_rows(void* out, const float* ws_o, const float* ws_ml, int rows, int H, int hd,
-                            int parts, void* stream) {
+                            int parts, const AttnExtras& ex, void* stream) {
   HE_REQUIRE(parts >= 1 && parts <= 64 && hd % 2 == 0, "he_attention_merge_rows: %d parts (at most 64), head_dim %d", parts, hd);
   const int64_t pairs = (int64_t)rows * H;
   HE_REQUIRE((pairs + 3) / 4 < (1ll << 31), "he_attention_merge_rows: too many rows for one launch");
   if (pairs == 0) return 0;
   attention_merge_rows_kernel<<<(unsigned)((pairs + 3) / 4), 256, 0, (hipStream_t)stream>>>(
-      (uint16_t*)out, ws_o, ws_ml, pairs, hd, parts);
+      (uint16_t*)out, ws_o, ws_ml, pairs, hd, parts, H, ex);
   return he_check_launch("he_attention_merge_rows");
 }
 
@@ -397,7 +404,8 @@ int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, c
                              int rows, int H, int hd, int parts, int out_pieces, void* stream) {
   HE_REQUIRE(parts >= 1 && parts <= 64, "he_attention_merge_parts: %d parts, at most 64", parts);
   attention_merge_kernel<<<dim3(H, rows), 256, 0, (hipStream_t)stream>>>(
-      (uint16_t*)out, ws_o, ws_ml, nullptr, (const int32_t*)row_seq, H, hd, parts, 0, 1, out_pieces);
+      (uint16_t*)out, ws_o, ws_ml, nullptr, (const int32_t*)row_seq, H, hd, parts, 0, 1, out_pieces,
+      AttnExtras{nullptr, 0, nullptr, 0, 0});
   return he_check_launch("he_attention_merge_parts");
 }
 
@@ -432,7 +440,9 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
                                          int num_seqs, int max_q_len, int H, int KVH, int hd,
                                          int window, float scale, int kernel, int total_rows,
                                          int parts, void* workspace_f32, int64_t workspace_floats,
-                                         void* stream) {
+                                         int chunk, const void* sinks, int sinks_dtype,
+                                         const void* gate, int64_t gate_stride, void* stream) {
+  const AttnExtras ex = {sinks, sinks_dtype, (const uint16_t*)gate, gate_stride, chunk};
   HE_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && H > 0 && KVH > 0 && hd > 0 && total_rows >= 0,
              "he_attention_prefill_bf16: bad sizes");
   HE_REQUIRE(kernel >= 0 && kernel <= 2,
@@ -466,9 +476,9 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
     }
     int rc = he_attention_prefill_wide(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
                                        max_blocks, num_pages, num_seqs, max_q_len, H, KVH, hd, window, scale,
-                                       parts, ws_o, ws_ml, stream);
+                                       parts, ws_o, ws_ml, ex, stream);
     if (rc || parts == 1) return rc;
-    return he_attention_merge_rows(out, ws_o, ws_ml, total_rows, H, hd, parts, stream);
+    return he_attention_merge_rows(out, ws_o, ws_ml, total_rows, H, hd, parts, ex, stream);
   }
   dim3 grid((max_q_len + 63) / 64, H, num_seqs);
   ATTN_SWITCH(hd / 16, (attention_prefill_kernel<NT><<<grid, 256, 0, s>>>(
@@ -476,6 +486,6 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
                            (const uint16_t*)vpool, (const int32_t*)cu_seqlens,
                            (const int32_t*)seq_slot, (const int32_t*)seq_start,
                            (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window,
-                           scale)));
+                           scale, ex)));
   return he_check_launch("he_attention_prefill_bf16");
 }

@@ -343,7 +343,7 @@ attention_prefill_wide_kernel(
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ page_table, int max_blocks,
     int num_pages, int H, int KVH, int window, float scale, int parts, float* __restrict__ ws_o,
-    float* __restrict__ ws_ml) {
+    float* __restrict__ ws_ml, AttnExtras ex) {
   constexpr int HD = Pw<NT>::HD, KS = Pw<NT>::KS, DT = Pw<NT>::DT;
   constexpr int KP = Pw<NT>::K_PIECES, VP = Pw<NT>::V_PIECES;
   __shared__ uint4 k_lds[2 * KP];
@@ -392,7 +392,7 @@ attention_prefill_wide_kernel(
 
   // the workgroup's pages: from the first key its first query sees to its last query
   const int blk_last = start + min(q0 + PW_QUERIES, q_len) - 1;
-  const int blk_first = window > 0 ? max(0, start + q0 + 1 - window) : 0;
+  const int blk_first = attn_first(start + q0, window, ex.chunk);
   int pbA = blk_first >> HE_PAGE_SHIFT, pbB = blk_last >> HE_PAGE_SHIFT;
   if (parts > 1) {
     // this workgroup's share of the block's pages; one without pages leaves empty parts
@@ -416,7 +416,7 @@ attention_prefill_wide_kernel(
   }
   WideTile<NT> t;
   t.hi = start + qi;
-  t.lo = window > 0 ? max(0, t.hi + 1 - window) : 0;
+  t.lo = attn_first(t.hi, window, ex.chunk);
   t.m = -INFINITY;
   t.l = 0.f;
 #pragma unroll
@@ -430,8 +430,8 @@ attention_prefill_wide_kernel(
   }
   // steps of 32 keys (hs: keys 32hs..32hs+31) of the tile: hsA..hsB; without a mask: hsI0..hsI1-1
   const int first_pos = start + qt, last_pos = start + min(qt + 31, q_len - 1);
-  const int lo_min = window > 0 ? max(0, first_pos + 1 - window) : 0;
-  const int lo_max = window > 0 ? max(0, last_pos + 1 - window) : 0;
+  const int lo_min = attn_first(first_pos, window, ex.chunk);
+  const int lo_max = attn_first(last_pos, window, ex.chunk);
   // (a part has the steps of its own pages only)
   const int hsA = tile ? max(lo_min >> 5, 2 * pbA) : 1, hsB = tile ? min(last_pos >> 5, 2 * pbB + 1) : 0;
   const int hsI0 = (lo_max + 31) >> 5, hsI1 = (first_pos + 1) >> 5;
@@ -515,7 +515,9 @@ attention_prefill_wide_kernel(
       }
     return;
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  // the sink joins the sum, the gate scales the output (a step in parts leaves both to the join)
+  const float lsum = l + attn_sink_term(ex, h, t.m);
+  const float inv = (lsum > 0.f ? 1.f / lsum : 0.f) * attn_gate(ex, row0 + qi, h);
   uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD + 4 * g;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -533,7 +535,7 @@ int he_attention_prefill_wide(void* out, const void* q, const void* kpool, const
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,
                               const void* page_table, int max_blocks, int num_pages, int num_seqs,
                               int max_q_len, int H, int KVH, int hd, int window, float scale,
-                              int parts, float* ws_o, float* ws_ml, void* stream) {
+                              int parts, float* ws_o, float* ws_ml, const AttnExtras& ex, void* stream) {
   HE_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 128,
              "he_attention_prefill_wide: head_dim %d must be a multiple of 16 up to 128", hd);
   HE_REQUIRE(parts >= 1 && parts <= 64 && (parts == 1 || (ws_o != nullptr && ws_ml != nullptr)),
@@ -548,7 +550,7 @@ int he_attention_prefill_wide(void* out, const void* q, const void* kpool, const
         (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,     \
         (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, (const int32_t*)seq_start,        \
         (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale, parts, ws_o,  \
-        ws_ml);                                                                                 \
+        ws_ml, ex);                                                                             \
     break;
   switch (hd / 16) {
     PREFILL_WIDE(1) PREFILL_WIDE(2) PREFILL_WIDE(3) PREFILL_WIDE(4)

@@ -11,6 +11,24 @@
 // queries of a tile move it in most steps, and every move rescales all accumulators.
 #define HE_SOFTMAX_SLACK 8.0f
 
+// (struct AttnExtras: common.h)
+// the first key the query at position pos sees (not decreasing in pos)
+__device__ __forceinline__ int attn_first(int pos, int window, int chunk) {
+  int first = window > 0 ? max(0, pos + 1 - window) : 0;
+  if (chunk > 0) first = max(first, pos - pos % chunk);
+  return first;
+}
+// the sink's share of the sum whose reference point is m (base-2 domain); 0 without sinks
+__device__ __forceinline__ float attn_sink_term(const AttnExtras& ex, int h, float m) {
+  if (ex.sinks == nullptr || !(m > -INFINITY)) return 0.f;
+  return __builtin_amdgcn_exp2f(load_param(ex.sinks, h, ex.sinks_dtype) * 1.4426950408889634f - m);
+}
+__device__ __forceinline__ float attn_gate(const AttnExtras& ex, int64_t row, int h) {
+  if (ex.gate == nullptr) return 1.f;
+  const float g = bf16_bits_to_float(ex.gate[row * ex.gate_stride + h]);
+  return 1.f / (1.f + __expf(-g));
+}
+
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 

@@ -196,6 +196,18 @@ void he_set_error(const char* fmt, ...);
 int he_check_launch(const char* what);
 // compute units of the current device (errors.hip); the host-side plans count in them
 int he_cus();
+// What an attention kernel may be asked for beyond the causal mask and the window, each off at its
+// null or zero: chunk > 0, a query sees no key before the start of its own chunk of that many
+// positions (counted from position 0); sinks, a number a head that joins the softmax's denominator
+// as exp(sink) without a key or value (not scaled); gate, gate[row * gate_stride + h] (bf16), whose
+// sigmoid multiplies the head's output.
+struct AttnExtras {
+  const void* sinks;
+  int sinks_dtype;
+  const uint16_t* gate;
+  int64_t gate_stride;
+  int chunk;
+};
 // attention_mfma.hip: joins attention parts that were all stored (the fused one-token kernel's, the
 // prompt kernel's); row_seq may be null: every row has a sequence
 int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,
@@ -208,7 +220,7 @@ int he_attention_prefill_wide(void* out, const void* q, const void* kpool, const
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,
                               const void* page_table, int max_blocks, int num_pages, int num_seqs,
                               int max_q_len, int H, int KVH, int hd, int window, float scale,
-                              int parts, float* ws_o, float* ws_ml, void* stream);
+                              int parts, float* ws_o, float* ws_ml, const AttnExtras& ex, void* stream);
 
 #define HE_REQUIRE(cond, ...)      \
   do {                             \

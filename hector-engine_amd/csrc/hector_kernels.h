@@ -147,12 +147,15 @@ int he_attention_plain(void* out, const void* q, const void* kpool, const void* 
                        int KVH, int hd, int window, int chunk, float scale, const void* sinks,
                        int sinks_dtype, const void* gate, int64_t gate_stride, int dtype,
                        int most_keys, void* workspace_f32, int64_t workspace_floats, void* stream);
-// bf16, one query row per sequence (decode): split over the keys, then merged.
+// bf16, one query row per sequence (decode): split over the keys, then merged. chunk, sinks and
+// gate (bf16 here) as he_attention_plain takes them; so does he_attention_prefill_bf16.
 int he_attention_decode_bf16(void* out, const void* q, const void* kpool, const void* vpool,
                              const void* positions, const void* row_seq, const void* seq_slot,
                              const void* page_table, int max_blocks, int num_pages, int rows,
                              int H, int KVH, int hd, int window, float scale, int max_keys,
-                             void* workspace_f32, int64_t workspace_floats, void* stream);
+                             void* workspace_f32, int64_t workspace_floats, int chunk,
+                             const void* sinks, int sinks_dtype, const void* gate, int64_t gate_stride,
+                             void* stream);
 int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd, int max_keys);
 // bf16, one query row per sequence, one launch for bias + rotary + cache write + attention +
 // merge (a second launch joins the parts where few sequences are cut across workgroups).
@@ -192,7 +195,8 @@ int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const
                               const void* page_table, int max_blocks, int num_pages, int num_seqs,
                               int max_q_len, int H, int KVH, int hd, int window, float scale,
                               int kernel, int total_rows, int parts, void* workspace_f32,
-                              int64_t workspace_floats, void* stream);
+                              int64_t workspace_floats, int chunk, const void* sinks, int sinks_dtype,
+                              const void* gate, int64_t gate_stride, void* stream);
 
 // ---- sampling ------------------------------------------------------------
 int64_t he_argmax_workspace_bytes(int rows, int V);

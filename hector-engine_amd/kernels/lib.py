@@ -61,7 +61,7 @@ _SIGNATURES = {
                            c_int, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_decode_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr,
-                                 c_i64, c_ptr],
+                                 c_i64, c_int, c_ptr, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_decode_workspace_floats": [c_int, c_int, c_int, c_int, c_int],
     "he_attention_decode_fused_ok": [c_int, c_int, c_int, c_int],
     "he_attention_decode_fused_workspace_floats": [c_int, c_int, c_int, c_int, c_int, c_int],
@@ -70,7 +70,7 @@ _SIGNATURES = {
                                        c_int, c_int, c_f32, c_int, c_int, c_int, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_prefill_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int,
-                                  c_int, c_int, c_ptr, c_i64, c_ptr],
+                                  c_int, c_int, c_ptr, c_i64, c_int, c_ptr, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_prefill_parts": [c_int, c_int, c_int, c_int, c_int],
     "he_attention_prefill_workspace_floats": [c_int, c_int, c_int, c_int],
     "he_argmax_workspace_bytes": [c_int, c_int],

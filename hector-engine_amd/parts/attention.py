@@ -176,7 +176,7 @@ class Attention(Mixer):
         if route is None:
             rot = self.position.rotary()
             case = AttentionCase(
-                all_single=ctx.all_single, fast=self.fast and not self.extras,
+                all_single=ctx.all_single, fast=self.fast,
                 fusable=not self.position.custom and rot is not None and not self.extras
                 and self.hd == self.vd == self.pd
                 and not self.position.interleaved and self.position.mscale == 1.0
@@ -254,24 +254,26 @@ class Attention(Mixer):
     def _run_mfma_one_token(self, x, ctx: StepContext, cache: LayerCache):
         """One-token steps of the head sizes and encodings the fused kernel does not take."""
         rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.pd
-        q, _ = self._encoded_q(x, ctx, cache)
+        q, gate = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
         floats = ops.attention_decode_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
         ws = ctx.alloc((max(floats, 1),), torch.float32)
         ops.attention_decode(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                              ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                             self.scale, ctx.max_keys, ws)
+                             self.scale, ctx.max_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate)
         return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
 
     def _run_mfma_prompt(self, x, ctx: StepContext, cache: LayerCache):
         """Prompt steps and mixed steps."""
         rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.pd
-        q, _ = self._encoded_q(x, ctx, cache)
+        q, gate = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
         # few queries against many keys (a continuation of a long sequence): the keys in parts
         most = ctx.most_keys
         if self.window > 0:
             most = min(most, self.window + ctx.max_q_len)
+        if self.chunk > 0:
+            most = min(most, self.chunk + ctx.max_q_len)
         parts = ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
         ws = ctx.alloc((ops.attention_prefill_workspace_floats(rows, H, hd, parts),), torch.float32) \
             if parts > 1 else None
@@ -281,7 +283,8 @@ class Attention(Mixer):
             (ws if ws is not None else out).zero_()
         ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
                               ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
-                              rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws)
+                              rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws,
+                              chunk=self.chunk, sinks=self.sinks, gate=gate)
         return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
 
 
