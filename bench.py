@@ -4,6 +4,7 @@ token ids) on one MI355X, with prefill and roofline figures on the same line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b|32b|72b]
                     [--context C] [--prompt P]
+    python bench.py --design volonex      (another measurement: see below)
 
 The default is the 7B shape; --shape runs the same measurement at the layer sizes of
 Qwen2.5-32B (context 8192, prompts of 512 to 2048 tokens, batches 1 / 8 / 64) or
@@ -26,6 +27,13 @@ The default warm-up of 64 steps is most of the first half second after the promp
 the machine runs every kernel of the one-token step 4 to 6 % slower than afterwards (the reference
 leaves its first run and its thermal-low samples out: OPTIMIZATION_NOTES.md:114-117); `repeats` holds
 every timed run, the earlier ones still show it.
+
+--design volonex leaves the run above aside and measures the Volonex design beside Qwen2 at equal layer
+sizes (random weights, bf16, four layers of each of a few sizes that resemble real models' layers): prompt
+tokens a second for one prompt of 2,048 tokens, decoded tokens a second at batch 8 and batch 1 behind such
+prompts, and, from a second pass with an event pair around every launch, the mean time of each kind of
+kernel in the prompt step and in the one-token step of both designs side by side. One JSON line,
+`"metric": "design_comparison"`.
 
 Procedure (the reference quotes medians with their range over repeated runs:
 tools/HQS_DECODE_OPTIMIZATION_PLAN.md:54-65): after the warm-up steps, `--repeats` (5) runs of
@@ -84,6 +92,125 @@ def prefill_flops(c, layers, T):
     return layers * (gemm + attn) + 2 * D * V
 
 
+# layer sizes of the design comparison: width, heads, kv heads, key width, value width, feed-forward
+DESIGN_SIZES = {
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, ff=8192),
+    "w3584": dict(width=3584, heads=28, kv_heads=4, dim=128, vdim=128, ff=18944),
+    "w4096_k64_v128": dict(width=4096, heads=32, kv_heads=8, dim=64, vdim=128, ff=14336),
+}
+DESIGN_LAYERS, DESIGN_VOCAB, DESIGN_CONTEXT = 4, 32000, 4096
+
+
+def design_configs(sz):
+    """(Qwen2 configuration, Volonex configuration) of one set of layer sizes. Where the Volonex layer has
+    keys and values of different widths, the Qwen2 layer has heads of the wider of the two."""
+    from hector_engine_amd.registry import config_from_dict
+    hd = max(sz["dim"], sz["vdim"])
+    qwen = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=DESIGN_LAYERS, hidden_size=sz["width"],
+                num_attention_heads=sz["heads"], num_key_value_heads=sz["kv_heads"], head_dim=hd,
+                intermediate_size=sz["ff"], vocab_size=DESIGN_VOCAB, rope_theta=1000000.0, rms_norm_eps=1e-6,
+                max_position_embeddings=DESIGN_CONTEXT, tie_word_embeddings=False)
+    mixer = dict(dim=sz["dim"], vdim=sz["vdim"], heads=sz["heads"], kv_heads=sz["kv_heads"],
+                 scale=sz["dim"] ** -0.5, mask=dict(size=2048),
+                 rot=dict(base=1000000.0, dims=sz["dim"] // 2,
+                          scaling=dict(factor=4.0, original=1024, fast=32.0, slow=1.0)))
+    layer = dict(type="attention", mixer=mixer, mlp=dict(kind="dense", ff=sz["ff"], limit=7.0))
+    volonex = dict(architecture="Volonex", vocab=DESIGN_VOCAB, width=sz["width"], residual_mult=0.5,
+                   embedding=dict(scale=1.0), norm=dict(eps=1e-6), layers=[layer] * DESIGN_LAYERS,
+                   loop=dict(start=0, stop=0, times=1))
+    return config_from_dict(qwen), config_from_dict(volonex)
+
+
+def compare_designs(args) -> int:
+    import torch
+    import hector_engine_amd as he
+    from hector_engine_amd.engine.engine import StepEntry
+
+    t_start = time.perf_counter()
+
+    def progress(what):
+        print(f"[bench {time.perf_counter() - t_start:6.1f}s] {what}", file=sys.stderr, flush=True)
+
+    rng = np.random.default_rng(0)
+    prompt_len, batch, steps = PROMPT, args.batch, min(args.steps, 64)
+
+    def measure(config, profile):
+        eng = he.Engine(config=config, seed=0, dtype="bfloat16", max_tokens=(batch + 1) * DESIGN_CONTEXT,
+                        max_slots=batch + 1, max_seq_len=DESIGN_CONTEXT, profile=profile, tune_library=not args.no_tune)
+        sampler = he.Sampler(he.SamplingConfig.deterministic(), eng.device)
+        ps = [rng.integers(0, DESIGN_VOCAB, prompt_len).tolist() for _ in range(batch)]
+        out = {}
+        # the prompt step: warm, captured, then timed
+        times = []
+        for run in range(5 if not profile else 2):
+            slot = eng.acquire()
+            if profile and run == 1:
+                eng.profiler.clear()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            eng.step([StepEntry(slot, ps[0], [prompt_len - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            eng.release(slot)
+        if profile:
+            eng.profiler.collect()
+            out["prefill_kernels_us"] = {name: round(1000 * avg, 1) for name, calls, total, avg, pct in eng.profiler.rows()}
+        else:
+            out["prefill_tok_s"] = round(prompt_len / sorted(times[2:])[1], 1)
+        for b in ([batch, 1] if not profile else [batch]):
+            slots = [eng.acquire() for _ in range(b)]
+            toks = []
+            for s, p in zip(slots, ps):
+                toks += sampler.sample(eng.step([StepEntry(s, p, [prompt_len - 1])]), [0], [0])
+            seqs = list(range(b))
+
+            def many(toks, count):
+                ids, reads = None, []
+                for j in range(count):
+                    logits = eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)], device_tokens=ids)
+                    ids = sampler.sample_device(logits, seqs, [0] * b)
+                    reads.append(sampler.read_later(ids))
+                    if j >= RUN - 1:
+                        reads[j - (RUN - 1)].wait()
+                return reads[-1].wait()
+
+            toks = many(toks, 8 if profile else args.warmup)
+            if profile:
+                eng.profiler.clear()
+                many(toks, 8)
+                eng.profiler.collect()
+                out["decode_kernels_us"] = {name: round(1000 * avg, 1) for name, calls, total, avg, pct in eng.profiler.rows()}
+            else:
+                runs = []
+                for _ in range(3):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    toks = many(toks, steps)
+                    torch.cuda.synchronize()
+                    runs.append((time.perf_counter() - t0) / steps)
+                out[f"decode_b{b}_tok_s"] = round(b / sorted(runs)[1], 1)
+                out[f"decode_b{b}_ms"] = round(1000 * sorted(runs)[1], 3)
+            for s in slots:
+                eng.release(s)
+        if eng.capture_failures:
+            raise RuntimeError(f"bench.py: steps ran without their graph: {eng.capture_failures}")
+        del eng, sampler
+        torch.cuda.empty_cache()
+        return out
+
+    result = {}
+    for name, sz in DESIGN_SIZES.items():
+        result[name] = {"sizes": sz}
+        for design, config in zip(("qwen2", "volonex"), design_configs(sz)):
+            progress(f"{name} {design}")
+            result[name][design] = measure(config, False)
+            result[name][design].update(measure(config, True))
+    print(json.dumps({"metric": "design_comparison", "design": "volonex", "beside": "qwen2", "dtype": "bf16",
+                      "data": "synthetic", "layers": DESIGN_LAYERS, "vocab": DESIGN_VOCAB, "prompt": prompt_len,
+                      "batch": batch, "steps": steps, "sizes": result}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -113,7 +240,12 @@ def main() -> int:
                     help="float32: the whole measurement in true 32-bit (no library products, no extra points)")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
+    ap.add_argument("--design", choices=["volonex"], default=None,
+                    help="instead of the run above: this design beside Qwen2 at equal layer sizes, prompt and "
+                         "one-token steps, throughput and mean time per kind of kernel")
     args = ap.parse_args()
+    if args.design:
+        return compare_designs(args)
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2

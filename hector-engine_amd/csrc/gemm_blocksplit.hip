@@ -124,6 +124,7 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
                                              float scale_eps, void* resid, const void* gain,
                                              int gain_dtype, void* xg, void* sq_out,
                                              int sq_count, int x_pieces, int out_pieces,
+                                             float act_alpha, float act_limit, float act_shift,
                                              void* stream) {
   HE_REQUIRE(M > 0 && M <= HE_BLOCKSPLIT_MAX_M, "he_gemm_blocksplit_bf16: M=%d outside [1, %d]", M,
              HE_BLOCKSPLIT_MAX_M);
@@ -165,6 +166,10 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
   fu.xg = (uint16_t*)xg;
   fu.sq_out = (float*)sq_out;
   fu.out_pieces = out_pieces;
+  fu.act_clamped = gated && !(act_alpha == 1.f && !(act_limit > 0.f) && act_shift == 0.f);
+  fu.act.alpha = act_alpha;
+  fu.act.limit = act_limit > 0.f ? act_limit : INFINITY;
+  fu.act.shift = act_shift;
   hipStream_t s = (hipStream_t)stream;
   int rc;
   static int (*const tiles[2][2])(HE_BS_DISPATCH_ARGS) = {
@@ -180,5 +185,5 @@ extern "C" int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, co
                                        int gated, int R, int U, int NW, void* stream) {
   return he_gemm_blocksplit_fused_bf16(C, A, W, bias, M, N, K, out_dtype, bias_dtype, gated, R, U,
                                        NW, nullptr, 0, 0.f, nullptr, nullptr, HE_F32, nullptr,
-                                       nullptr, 0, 0, 0, stream);
+                                       nullptr, 0, 0, 0, 1.f, 0.f, 0.f, stream);
 }

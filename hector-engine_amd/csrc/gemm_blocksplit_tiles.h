@@ -152,6 +152,8 @@ struct BsFusion {
   uint16_t* xg;                  // [M][N] bf16 out: resid * gain
   float* sq_out;                 // [M][gridDim.x] out: sum of resid^2 over this workgroup's columns
   int out_pieces;                // the bf16 output (C, or xg) is written piece-major
+  int act_clamped;               // the gated epilogue runs he_gated_act with `act`, not SiLU(gate) * up
+  GatedAct act;
 };
 
 // The residual values and gains of output item (tile, lane) of a non-gated product:
@@ -356,7 +358,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const float g = v[2 * i] * rs;
-        y[i] = g / (1.f + expf(-g)) * (v[2 * i + 1] * rs);
+        y[i] = fu.act_clamped ? he_gated_act<true>(g, v[2 * i + 1] * rs, fu.act)
+                              : g / (1.f + expf(-g)) * (v[2 * i + 1] * rs);
       }
       if (fu.out_pieces)
         bs_store_pieces(reinterpret_cast<uint16_t*>(C), M, m, n >> 1, y, 2, valid);

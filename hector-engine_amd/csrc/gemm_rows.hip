@@ -85,7 +85,7 @@ extern "C" int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_flo
                                  const void* scale_partials, int scale_count, float scale_eps,
                                  void* resid, const void* gain, int gain_dtype, void* xg, void* sq_out,
                                  int sq_count, int x_pieces, int out_pieces, int* splits_used,
-                                 void* stream) {
+                                 float act_alpha, float act_limit, float act_shift, void* stream) {
   HE_REQUIRE(M > 0 && M <= HE_GEMM_ROWS_MAX_M, "he_gemm_rows_bf16: M=%d outside [1, %d]", M,
              HE_GEMM_ROWS_MAX_M);
   HE_REQUIRE(N > 0 && K > 0, "he_gemm_rows_bf16: bad sizes N=%d K=%d", N, K);
@@ -133,6 +133,10 @@ extern "C" int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_flo
   fu.xg = (uint16_t*)xg;
   fu.sq_out = (float*)sq_out;
   fu.out_pieces = out_pieces;
+  fu.act_clamped = gated && !(act_alpha == 1.f && !(act_limit > 0.f) && act_shift == 0.f);
+  fu.act.alpha = act_alpha;
+  fu.act.limit = act_limit > 0.f ? act_limit : INFINITY;
+  fu.act.shift = act_shift;
   hipStream_t s = (hipStream_t)stream;
   float* partial = (float*)partial_f32;
   int rc;

@@ -22,6 +22,8 @@ struct RowsFusion {
   uint16_t* xg;                  // [M][N] bf16 out: resid * gain
   float* sq_out;                 // [M][gridDim.x] out: sum of resid^2 over this workgroup's columns
   int out_pieces;                // the bf16 output (C, or xg) is written piece-major
+  int act_clamped;               // the gated epilogue runs he_gated_act with `act`, not SiLU(gate) * up
+  GatedAct act;
 };
 
 template <int R>
@@ -323,7 +325,9 @@ __global__ __launch_bounds__(64 * NWV) void gemm_rows_kernel(
         const int NO = N >> 1;
         float y[2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) y[i] = v[2 * i] / (1.f + expf(-v[2 * i])) * v[2 * i + 1];
+        for (int i = 0; i < 2; ++i)
+          y[i] = fu.act_clamped ? he_gated_act<true>(v[2 * i], v[2 * i + 1], fu.act)
+                                : v[2 * i] / (1.f + expf(-v[2 * i])) * v[2 * i + 1];
         if (fu.out_pieces)
           rows_store_pieces(reinterpret_cast<uint16_t*>(C), M, m, n >> 1, y, 2, valid >> 1);
         else if (((NO | (n >> 1)) & 1) == 0 && valid == 4) {

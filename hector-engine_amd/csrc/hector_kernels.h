@@ -84,7 +84,9 @@ int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void* W, const v
                                   int U, int NW, const void* scale_partials, int scale_count,
                                   float scale_eps, void* resid, const void* gain, int gain_dtype,
                                   void* xg, void* sq_out, int sq_count, int x_pieces, int out_pieces,
-                                  void* stream);
+                                  float act_alpha, float act_limit, float act_shift, void* stream);
+// act_alpha, act_limit, act_shift: the constants of the gated epilogue as he_gated_act takes them
+// (1, 0, 0: SiLU(gate) * up); so for he_gemm_rows_bf16.
 // out = x / sqrt(sum(partials of the row)/D + eps): such xg rows as a normalised tensor
 // (row-major; x_pieces: x lies piece-major for exactly `rows` rows).
 int he_scale_rows_bf16(void* out, const void* x, const void* partials, int count, int rows, int D,
@@ -106,7 +108,7 @@ int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_floats, const 
                       int R, int NWV, int splits, const void* scale_partials, int scale_count,
                       float scale_eps, void* resid, const void* gain, int gain_dtype, void* xg,
                       void* sq_out, int sq_count, int x_pieces, int out_pieces, int* splits_used,
-                      void* stream);
+                      float act_alpha, float act_limit, float act_shift, void* stream);
 // resid[M,N] (fp32, in place) += the slices of partial_f32 [splits][M][N] in index order (+ bias);
 // xg = bf16(resid * gain) (piece-major with out_pieces); sq_out[M, sq_count] = sums of resid^2 per
 // block of 1024 columns (sq_count = he_splitk_reduce_residual_blocks(N)): the rows a residual

@@ -261,11 +261,13 @@ def gemm_blocksplit_blocks(M: int, N: int, K: int) -> int:
 
 @_op("gemm_blocksplit")
 def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0), *,
-                    row_scale=None, residual=None, x_pieces: bool = False, out_pieces: bool = False) -> None:
+                    row_scale=None, residual=None, x_pieces: bool = False, out_pieces: bool = False,
+                    act=(1.0, 0.0, 0.0)) -> None:
     """bf16 MFMA product for M <= 32 with K cut inside the workgroup; one launch, complete
     result (bf16 or fp32), with bias or, gated, as [M, N/2] = silu(gate) * up for a weight
     that alternates gate and up rows (gate i at row 2i, its up at 2i + 1). plan = (R, U, NW),
-    zeros = heuristic.
+    zeros = heuristic. act = (alpha, limit, up_shift): the gated epilogue's constants as silu_mul
+    takes them.
 
     row_scale = (partials fp32 [M, count], eps): the rows of `a` are r * gain of an RMS norm
     whose 1/sqrt(mean(r^2) + eps) is applied to the sums here (mean over K).
@@ -324,7 +326,7 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
         dtype_code(out.dtype) if out is not None else BF16,
         dtype_code(bias.dtype) if bias is not None else F32, int(gated),
         int(plan[0]), int(plan[1]), int(plan[2]), sp, sc, float(se), rp, gp, gdt, xp, qp, qc,
-        int(x_pieces), int(out_pieces), _stream()))
+        int(x_pieces), int(out_pieces), float(act[0]), float(act[1]), float(act[2]), _stream()))
 
 
 def gemm_rows_plan(M: int, N: int, K: int) -> tuple[int, int]:
@@ -338,7 +340,7 @@ def gemm_rows_plan(M: int, N: int, K: int) -> tuple[int, int]:
 
 @_op("gemm_rows")
 def gemm_rows(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0), *, row_scale=None,
-              residual=None, x_pieces: bool = False, out_pieces: bool = False) -> int:
+              residual=None, x_pieces: bool = False, out_pieces: bool = False, act=(1.0, 0.0, 0.0)) -> int:
     """bf16 MFMA product for M <= 64 whose activation rows go through LDS once per workgroup; the
     epilogues of gemm_blocksplit (see there: bias, gated, row_scale, residual, x_pieces, out_pieces).
     plan = (R, NWV, splits), zeros = heuristic. A product cut into several K slices writes its fp32
@@ -396,7 +398,8 @@ def gemm_rows(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 0,
         dtype_code(out.dtype) if out is not None else BF16,
         dtype_code(bias.dtype) if bias is not None else F32, int(gated),
         int(plan[0]), int(plan[1]), int(plan[2]), sp, sc, float(se), rp, gp, gdt, xp, qp, qc,
-        int(x_pieces), int(out_pieces), ctypes.byref(used), _stream()))
+        int(x_pieces), int(out_pieces), ctypes.byref(used), float(act[0]), float(act[1]), float(act[2]),
+        _stream()))
     return used.value
 
 

@@ -278,28 +278,31 @@ class Linear:
         return self._has("gated", rows, ctx, act) and self.weight.shape[0] % 2 == 0
 
     def gated_silu(self, x, rows: int, ctx: StepContext, out: torch.Tensor,
-                   out_pieces: bool = False) -> None:
+                   out_pieces: bool = False, act: dict | None = None) -> None:
         """out[rows, N/2] = silu(gate) * up in one kernel, for a weight whose rows alternate gate
         and up (gate i at row 2i, its up at 2i + 1), where gated_silu_rows() says so. x: a tensor,
-        NormedRows or PieceRows; out_pieces: out is shaped and written piece-major."""
+        NormedRows or PieceRows; out_pieces: out is shaped and written piece-major. act: the
+        constants of another gated activation ({alpha, limit, up_shift} as ops.silu_mul takes them)."""
+        act = act or {}
+        consts = (act.get("alpha", 1.0), act.get("limit", 0.0), act.get("up_shift", 0.0))
         act, a, scale, pieces = _operand(x)
         if not self.gated_silu_rows(rows, ctx, act):
             raise ValueError("Linear.gated_silu: not for these rows (ask gated_silu_rows)")
         if rows <= ops.BLOCKSPLIT_PIECES_MAX_M:
             ops.gemm_blocksplit(out, a, self.weight, None, rows, gated=True, row_scale=scale,
-                                x_pieces=pieces, out_pieces=out_pieces)
+                                x_pieces=pieces, out_pieces=out_pieces, act=consts)
             return
         splits = self._plan(rows)[1]
         if splits == 1:
             ops.gemm_rows(out, None, a, self.weight, None, rows, gated=True, row_scale=scale,
-                          x_pieces=pieces, out_pieces=out_pieces)
+                          x_pieces=pieces, out_pieces=out_pieces, act=consts)
             return
         # few weight rows, cut along K: the activation kernel adds the slices while it reads them
         if out_pieces:
             raise ValueError("Linear.gated_silu: a product cut along K writes row-major (ask gated_pieces)")
         partial = ctx.alloc((splits, rows, self.weight.shape[0]), torch.float32)
         ops.gemm_rows(None, partial, a, self.weight, None, rows, row_scale=scale, x_pieces=pieces)
-        ops.silu_mul(out, partial, rows, True, splits)
+        ops.silu_mul(out, partial, rows, True, splits, **act)
 
     def gated_pieces(self, rows: int) -> bool:
         """Whether gated_silu can write its result piece-major at this many rows."""

@@ -70,12 +70,12 @@ class GatedMLP(FeedForward):
         rows = ctx.rows
         if rows <= _ROW_CHUNK:
             act = x.scaled.dtype if isinstance(x, NormedRows) else x.dtype
-            if not self.act and self.gate_up.gated_silu_rows(rows, ctx, act):
+            if self.gate_up.gated_silu_rows(rows, ctx, act):
                 # up to 64 rows: the activation is the product's epilogue, and its result goes to the
                 # down projection piece-major where that reads it so
                 pieces = self.inter % 8 == 0 and self.down.reads_pieces(rows, ctx) and self.gate_up.gated_pieces(rows)
                 h = ctx.alloc(ops.pieces_shape(rows, self.inter) if pieces else (rows, self.inter))
-                self.gate_up.gated_silu(x, rows, ctx, h, out_pieces=pieces)
+                self.gate_up.gated_silu(x, rows, ctx, h, out_pieces=pieces, act=self.act)
                 return self.down(PieceRows(h) if pieces else h, rows, ctx, sink=ctx.take_sink())
             h = ctx.alloc((rows, self.inter))
             gu = self.gate_up(x, rows, ctx)
