@@ -191,6 +191,20 @@ __device__ __forceinline__ float he_gated_act(float g, float u, const GatedAct& 
   return g / (1.f + expf(-a.alpha * g)) * (u + a.shift);
 }
 
+// tanh for a result that is rounded to bfloat16: (1 - t) / (1 + t) with t = exp(-2 |z|), the sign put back
+// (relative error below 1e-4 from |z| = 1e-3 on, far inside a bfloat16's half ulp of 2e-3).
+__device__ __forceinline__ float he_tanh_bf16(float z) {
+  const float t = __expf(-2.f * fabsf(z));
+  return copysignf((1.f - t) / (1.f + t), z);
+}
+// What a product's residual epilogue leaves for the norm that follows, from the new residual value x:
+// x * gain (an RMS norm, whose row scale the next product applies), or, with dyt_alpha, Dynamic Tanh in
+// full: tanh(alpha x) * gain + bias.
+__device__ __forceinline__ float he_carried_norm(float x, float gain, const void* dyt_bias, int n, int dtype,
+                                                 bool dyt, float alpha) {
+  return dyt ? fmaf(he_tanh_bf16(alpha * x), gain, load_param(dyt_bias, n, dtype)) : x * gain;
+}
+
 // ---- error channel -------------------------------------------------------
 void he_set_error(const char* fmt, ...);
 int he_check_launch(const char* what);

@@ -125,7 +125,9 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
                                              int gain_dtype, void* xg, void* sq_out,
                                              int sq_count, int x_pieces, int out_pieces,
                                              float act_alpha, float act_limit, float act_shift,
-                                             void* stream) {
+                                             float resid_scale, const void* dyt_bias,
+                                             const void* dyt_alpha, void* stream) {
+  HE_REQUIRE((dyt_alpha == nullptr) == (dyt_bias == nullptr), "he_gemm_blocksplit_bf16: Dynamic Tanh needs alpha and bias");
   HE_REQUIRE(M > 0 && M <= HE_BLOCKSPLIT_MAX_M, "he_gemm_blocksplit_bf16: M=%d outside [1, %d]", M,
              HE_BLOCKSPLIT_MAX_M);
   HE_REQUIRE(N > 0 && K > 0, "he_gemm_blocksplit_bf16: bad sizes N=%d K=%d", N, K);
@@ -170,6 +172,9 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
   fu.act.alpha = act_alpha;
   fu.act.limit = act_limit > 0.f ? act_limit : INFINITY;
   fu.act.shift = act_shift;
+  fu.resid_scale = resid_scale;
+  fu.dyt_bias = dyt_bias;
+  fu.dyt_alpha = dyt_alpha;
   hipStream_t s = (hipStream_t)stream;
   int rc;
   static int (*const tiles[2][2])(HE_BS_DISPATCH_ARGS) = {
@@ -185,5 +190,5 @@ extern "C" int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, co
                                        int gated, int R, int U, int NW, void* stream) {
   return he_gemm_blocksplit_fused_bf16(C, A, W, bias, M, N, K, out_dtype, bias_dtype, gated, R, U,
                                        NW, nullptr, 0, 0.f, nullptr, nullptr, HE_F32, nullptr,
-                                       nullptr, 0, 0, 0, 1.f, 0.f, 0.f, stream);
+                                       nullptr, 0, 0, 0, 1.f, 0.f, 0.f, 1.f, nullptr, nullptr, stream);
 }

@@ -154,6 +154,9 @@ struct BsFusion {
   int out_pieces;                // the bf16 output (C, or xg) is written piece-major
   int act_clamped;               // the gated epilogue runs he_gated_act with `act`, not SiLU(gate) * up
   GatedAct act;
+  float resid_scale;             // the residual epilogue adds resid_scale * result
+  const void* dyt_bias;          // with dyt_alpha: xg = tanh(alpha * resid) * gain + dyt_bias (Dynamic Tanh; both of
+  const void* dyt_alpha;         // gain's dtype; alpha one stored number), and sq_out = 0: nothing is owed
 };
 
 // The residual values and gains of output item (tile, lane) of a non-gated product:
@@ -240,6 +243,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   const int out_align = ((N | n0) & 3) == 0 ? 4 : (((N | n0) & 1) == 0 ? 2 : 1);
   const bool scaled = fu.scale_partials != nullptr;
   const bool to_resid = !GATED && fu.resid != nullptr;
+  const bool dyt = fu.dyt_alpha != nullptr;
+  const float dyt_a = dyt ? load_param(fu.dyt_alpha, 0, fu.gain_dtype) : 0.f;
   constexpr int SCALE_ROWS = 4;           // rows a wavefront takes: 16 rows with 4 wavefronts
   const bool scale_early = scaled && fu.scale_count <= 256 && M <= SCALE_ROWS * nw;
   float pv[SCALE_ROWS][4];
@@ -385,9 +390,9 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       float sq = 0.f, x[4], xgv[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        x[i] = res0[i] + v[i];
-        xgv[i] = x[i] * gain0[i];
-        if (i < valid) sq += x[i] * x[i];
+        x[i] = res0[i] + fu.resid_scale * v[i];
+        xgv[i] = he_carried_norm(x[i], gain0[i], fu.dyt_bias, min(n + i, N - 1), fu.gain_dtype, dyt, dyt_a);
+        if (i < valid && !dyt) sq += x[i] * x[i];
       }
       if (valid > 0) {
         const int64_t at = (int64_t)m * N + n;

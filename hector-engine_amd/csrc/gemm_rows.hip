@@ -85,7 +85,9 @@ extern "C" int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_flo
                                  const void* scale_partials, int scale_count, float scale_eps,
                                  void* resid, const void* gain, int gain_dtype, void* xg, void* sq_out,
                                  int sq_count, int x_pieces, int out_pieces, int* splits_used,
-                                 float act_alpha, float act_limit, float act_shift, void* stream) {
+                                 float act_alpha, float act_limit, float act_shift, float resid_scale,
+                                 const void* dyt_bias, const void* dyt_alpha, void* stream) {
+  HE_REQUIRE((dyt_alpha == nullptr) == (dyt_bias == nullptr), "he_gemm_rows_bf16: Dynamic Tanh needs alpha and bias");
   HE_REQUIRE(M > 0 && M <= HE_GEMM_ROWS_MAX_M, "he_gemm_rows_bf16: M=%d outside [1, %d]", M,
              HE_GEMM_ROWS_MAX_M);
   HE_REQUIRE(N > 0 && K > 0, "he_gemm_rows_bf16: bad sizes N=%d K=%d", N, K);
@@ -137,6 +139,9 @@ extern "C" int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_flo
   fu.act.alpha = act_alpha;
   fu.act.limit = act_limit > 0.f ? act_limit : INFINITY;
   fu.act.shift = act_shift;
+  fu.resid_scale = resid_scale;
+  fu.dyt_bias = dyt_bias;
+  fu.dyt_alpha = dyt_alpha;
   hipStream_t s = (hipStream_t)stream;
   float* partial = (float*)partial_f32;
   int rc;
@@ -222,8 +227,11 @@ extern "C" int he_splitk_reduce(void* C, const void* partial_f32, const void* bi
 __global__ __launch_bounds__(256) void splitk_reduce_residual_kernel(
     float* __restrict__ resid, const float* __restrict__ partial, const void* __restrict__ bias,
     int bias_dtype, const void* __restrict__ gain, int gain_dtype, uint16_t* __restrict__ xg,
-    float* __restrict__ sq_out, int M, int N, int splits, int out_pieces) {
+    float* __restrict__ sq_out, int M, int N, int splits, int out_pieces, float resid_scale,
+    const void* __restrict__ dyt_bias, const void* __restrict__ dyt_alpha) {
   __shared__ float red[4];
+  const bool dyt = dyt_alpha != nullptr;
+  const float dyt_a = dyt ? load_param(dyt_alpha, 0, gain_dtype) : 0.f;
   const int m = blockIdx.y;
   const int n = blockIdx.x * 1024 + 4 * threadIdx.x;
   float sq = 0.f;
@@ -259,9 +267,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_residual_kernel(
     for (int i = 0; i < 4; ++i) {
       const bool in = i < valid;
       if (in && bias != nullptr) d[i] += load_param(bias, n + i, bias_dtype);
-      x[i] += d[i];
-      g[i] = in ? x[i] * load_param(gain, n + i, gain_dtype) : 0.f;
-      if (in) sq += x[i] * x[i];
+      x[i] += resid_scale * d[i];
+      g[i] = in ? he_carried_norm(x[i], load_param(gain, n + i, gain_dtype), dyt_bias, n + i, gain_dtype, dyt, dyt_a) : 0.f;
+      if (in && !dyt) sq += x[i] * x[i];
     }
     if (vec) {
       *reinterpret_cast<float4*>(resid + at) = make_float4(x[0], x[1], x[2], x[3]);
@@ -287,7 +295,9 @@ extern "C" int he_splitk_reduce_residual_blocks(int N) { return N > 0 ? (N + 102
 extern "C" int he_splitk_reduce_residual(void* resid_f32, const void* partial_f32, const void* bias,
                                          int bias_dtype, const void* gain, int gain_dtype, void* xg,
                                          void* sq_out, int sq_count, int M, int N, int splits,
-                                         int out_pieces, void* stream) {
+                                         int out_pieces, float resid_scale, const void* dyt_bias,
+                                         const void* dyt_alpha, void* stream) {
+  HE_REQUIRE((dyt_alpha == nullptr) == (dyt_bias == nullptr), "he_splitk_reduce_residual: Dynamic Tanh needs alpha and bias");
   HE_REQUIRE(M >= 0 && M <= 65535 && N > 0 && splits > 0, "he_splitk_reduce_residual: bad sizes");
   HE_REQUIRE(resid_f32 && partial_f32 && gain && xg && sq_out, "he_splitk_reduce_residual: missing buffers");
   HE_REQUIRE(sq_count == he_splitk_reduce_residual_blocks(N),
@@ -299,6 +309,6 @@ extern "C" int he_splitk_reduce_residual(void* resid_f32, const void* partial_f3
   if (M == 0) return 0;
   splitk_reduce_residual_kernel<<<dim3(sq_count, M), 256, 0, (hipStream_t)stream>>>(
       (float*)resid_f32, (const float*)partial_f32, bias, bias_dtype, gain, gain_dtype, (uint16_t*)xg,
-      (float*)sq_out, M, N, splits, out_pieces);
+      (float*)sq_out, M, N, splits, out_pieces, resid_scale, dyt_bias, dyt_alpha);
   return he_check_launch("he_splitk_reduce_residual");
 }

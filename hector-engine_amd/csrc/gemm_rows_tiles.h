@@ -24,6 +24,9 @@ struct RowsFusion {
   int out_pieces;                // the bf16 output (C, or xg) is written piece-major
   int act_clamped;               // the gated epilogue runs he_gated_act with `act`, not SiLU(gate) * up
   GatedAct act;
+  float resid_scale;             // the residual epilogue adds resid_scale * result
+  const void* dyt_bias;          // with dyt_alpha: xg = tanh(alpha * resid) * gain + dyt_bias (Dynamic Tanh; both of
+  const void* dyt_alpha;         // gain's dtype; alpha one stored number), and sq_out = 0: nothing is owed
 };
 
 template <int R>
@@ -308,6 +311,8 @@ __global__ __launch_bounds__(64 * NWV) void gemm_rows_kernel(
   }
 
   const bool to_resid = !GATED && fu.resid != nullptr;
+  const bool dyt = fu.dyt_alpha != nullptr;
+  const float dyt_a = dyt ? load_param(fu.dyt_alpha, 0, fu.gain_dtype) : 0.f;
   float sq[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) sq[t] = 0.f;
@@ -354,9 +359,10 @@ __global__ __launch_bounds__(64 * NWV) void gemm_rows_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const bool in = i < valid;
-        x[i] = (in ? fu.resid[at + i] : 0.f) + v[i];
-        xgv[i] = in ? x[i] * load_param(fu.gain, n + i, fu.gain_dtype) : 0.f;
-        if (in) sq[t] += x[i] * x[i];
+        x[i] = (in ? fu.resid[at + i] : 0.f) + fu.resid_scale * v[i];
+        xgv[i] = in ? he_carried_norm(x[i], load_param(fu.gain, n + i, fu.gain_dtype), fu.dyt_bias, n + i,
+                                      fu.gain_dtype, dyt, dyt_a) : 0.f;
+        if (in && !dyt) sq[t] += x[i] * x[i];
       }
       rows_store4<float>(fu.resid + at, x, out_align, valid);
       if (fu.out_pieces)

@@ -84,7 +84,13 @@ int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void* W, const v
                                   int U, int NW, const void* scale_partials, int scale_count,
                                   float scale_eps, void* resid, const void* gain, int gain_dtype,
                                   void* xg, void* sq_out, int sq_count, int x_pieces, int out_pieces,
-                                  float act_alpha, float act_limit, float act_shift, void* stream);
+                                  float act_alpha, float act_limit, float act_shift, float resid_scale,
+                                  const void* dyt_bias, const void* dyt_alpha, void* stream);
+// resid_scale: the residual epilogue adds resid_scale * result. dyt_alpha, dyt_bias (both null, or both
+// of gain's dtype; alpha one stored number): the norm that follows is Dynamic Tanh, and the epilogue
+// leaves it finished, xg = tanh(alpha * resid) * gain + dyt_bias, with sq_out = 0 (a reader that
+// applies 1/sqrt(sum / K + eps) with eps = 1 applies 1). So for he_gemm_rows_bf16 and
+// he_splitk_reduce_residual.
 // act_alpha, act_limit, act_shift: the constants of the gated epilogue as he_gated_act takes them
 // (1, 0, 0: SiLU(gate) * up); so for he_gemm_rows_bf16.
 // out = x / sqrt(sum(partials of the row)/D + eps): such xg rows as a normalised tensor
@@ -108,7 +114,8 @@ int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_floats, const 
                       int R, int NWV, int splits, const void* scale_partials, int scale_count,
                       float scale_eps, void* resid, const void* gain, int gain_dtype, void* xg,
                       void* sq_out, int sq_count, int x_pieces, int out_pieces, int* splits_used,
-                      float act_alpha, float act_limit, float act_shift, void* stream);
+                      float act_alpha, float act_limit, float act_shift, float resid_scale,
+                      const void* dyt_bias, const void* dyt_alpha, void* stream);
 // resid[M,N] (fp32, in place) += the slices of partial_f32 [splits][M][N] in index order (+ bias);
 // xg = bf16(resid * gain) (piece-major with out_pieces); sq_out[M, sq_count] = sums of resid^2 per
 // block of 1024 columns (sq_count = he_splitk_reduce_residual_blocks(N)): the rows a residual
@@ -116,7 +123,8 @@ int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_floats, const 
 int he_splitk_reduce_residual_blocks(int N);
 int he_splitk_reduce_residual(void* resid_f32, const void* partial_f32, const void* bias, int bias_dtype,
                               const void* gain, int gain_dtype, void* xg, void* sq_out, int sq_count,
-                              int M, int N, int splits, int out_pieces, void* stream);
+                              int M, int N, int splits, int out_pieces, float resid_scale,
+                              const void* dyt_bias, const void* dyt_alpha, void* stream);
 
 // ---- position encoding + cache write -------------------------------------
 int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in, const void* k_in,

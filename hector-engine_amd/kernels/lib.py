@@ -42,16 +42,17 @@ _SIGNATURES = {
     "he_gemm_blocksplit_blocks": [c_int, c_int, c_int],
     "he_gemm_blocksplit_fused_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
                                       c_int, c_int, c_int, c_ptr, c_int, c_f32, c_ptr, c_ptr, c_int,
-                                      c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_f32, c_f32, c_ptr],
+                                      c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_f32, c_f32, c_f32, c_ptr, c_ptr,
+                                      c_ptr],
     "he_scale_rows_bf16": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_int, c_ptr],
     "he_splitk_reduce": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
     "he_gemm_rows_plan": [c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)],
     "he_gemm_rows_bf16": [c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
                           c_int, c_int, c_int, c_ptr, c_int, c_f32, c_ptr, c_ptr, c_int, c_ptr, c_ptr, c_int,
-                          c_int, c_int, ctypes.POINTER(c_int), c_f32, c_f32, c_f32, c_ptr],
+                          c_int, c_int, ctypes.POINTER(c_int), c_f32, c_f32, c_f32, c_f32, c_ptr, c_ptr, c_ptr],
     "he_splitk_reduce_residual_blocks": [c_int],
     "he_splitk_reduce_residual": [c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_int, c_int, c_int,
-                                  c_int, c_int, c_ptr],
+                                  c_int, c_int, c_f32, c_ptr, c_ptr, c_ptr],
     "he_qkv_rope_cache": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr,
                           c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr],

@@ -274,6 +274,9 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
     residual = (resid fp32 [M, N], gain [N], xg bf16 [M, N], sq fp32 [M, blocks]): instead of
     writing `out` (None), resid += result in place, xg = resid * gain, sq = the sums of resid^2
     per workgroup (blocks = gemm_blocksplit_blocks(M, N, K)).
+    The tuple may go on with (scale, dyt_bias, dyt_alpha): resid += scale * result, and with the last two
+    (a vector [N] and a one-element tensor of gain's dtype) the rows left are those of a Dynamic Tanh in
+    full, xg = tanh(alpha * resid) * gain + dyt_bias, and sq = 0 (with eps 1 nothing is owed).
     x_pieces: `a` is piece-major, shaped pieces_shape(M, K). out_pieces: the bf16 output (`out`,
     or xg of the residual epilogue) is written piece-major, shaped pieces_shape(M, its width)."""
     N, K = w.shape
@@ -307,8 +310,14 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
         sp, sc = partials.data_ptr(), partials.shape[1]
     rp = gp = xp = qp = None
     gdt, qc = F32, 0
+    rscale, dyt_bias, dyt_alpha = 1.0, None, None
     if residual is not None:
-        resid, gain, xg, sq = residual
+        resid, gain, xg, sq, *more = residual
+        rscale = more[0] if more else 1.0
+        dyt_bias, dyt_alpha = (more[1], more[2]) if len(more) > 2 else (None, None)
+        if dyt_alpha is not None:
+            _need(dyt_bias, "dyt bias", gain.dtype, (N,))
+            _need(dyt_alpha, "dyt alpha", gain.dtype)
         _need(resid, "resid", torch.float32)
         _need(gain, "gain", shape=(N,))
         _need(xg, "xg", torch.bfloat16)
@@ -326,7 +335,8 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
         dtype_code(out.dtype) if out is not None else BF16,
         dtype_code(bias.dtype) if bias is not None else F32, int(gated),
         int(plan[0]), int(plan[1]), int(plan[2]), sp, sc, float(se), rp, gp, gdt, xp, qp, qc,
-        int(x_pieces), int(out_pieces), float(act[0]), float(act[1]), float(act[2]), _stream()))
+        int(x_pieces), int(out_pieces), float(act[0]), float(act[1]), float(act[2]), float(rscale),
+        _ptr(dyt_bias), _ptr(dyt_alpha), _stream()))
 
 
 def gemm_rows_plan(M: int, N: int, K: int) -> tuple[int, int]:
@@ -378,8 +388,14 @@ def gemm_rows(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 0,
         sp, sc = partials.data_ptr(), partials.shape[1]
     rp = gp = xp = qp = None
     gdt, qc = F32, 0
+    rscale, dyt_bias, dyt_alpha = 1.0, None, None
     if residual is not None:
-        resid, gain, xg, sq = residual
+        resid, gain, xg, sq, *more = residual
+        rscale = more[0] if more else 1.0
+        dyt_bias, dyt_alpha = (more[1], more[2]) if len(more) > 2 else (None, None)
+        if dyt_alpha is not None:
+            _need(dyt_bias, "dyt bias", gain.dtype, (N,))
+            _need(dyt_alpha, "dyt alpha", gain.dtype)
         _need(resid, "resid", torch.float32)
         _need(gain, "gain", shape=(N,))
         _need(xg, "xg", torch.bfloat16)
@@ -399,7 +415,7 @@ def gemm_rows(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 0,
         dtype_code(bias.dtype) if bias is not None else F32, int(gated),
         int(plan[0]), int(plan[1]), int(plan[2]), sp, sc, float(se), rp, gp, gdt, xp, qp, qc,
         int(x_pieces), int(out_pieces), ctypes.byref(used), float(act[0]), float(act[1]), float(act[2]),
-        _stream()))
+        float(rscale), _ptr(dyt_bias), _ptr(dyt_alpha), _stream()))
     return used.value
 
 
@@ -409,7 +425,7 @@ def splitk_reduce_residual_blocks(N: int) -> int:
 
 @_op("splitk_reduce_residual")
 def splitk_reduce_residual(resid, partial, bias, gain, xg, sq, M: int, splits: int,
-                           out_pieces: bool = False) -> None:
+                           out_pieces: bool = False, *, scale: float = 1.0, dyt_bias=None, dyt_alpha=None) -> None:
     """resid [M, N] (fp32, in place) += the K slices partial [splits, M, N] in index order (+ bias);
     xg = bf16(resid * gain), piece-major with out_pieces; sq [M, blocks] = sums of resid^2 per block
     of columns (blocks = splitk_reduce_residual_blocks(N))."""
@@ -430,7 +446,7 @@ def splitk_reduce_residual(resid, partial, bias, gain, xg, sq, M: int, splits: i
     _lib.check(L.he_splitk_reduce_residual(
         resid.data_ptr(), partial.data_ptr(), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
         gain.data_ptr(), dtype_code(gain.dtype), xg.data_ptr(), sq.data_ptr(), sq.shape[1], M, N, splits,
-        int(out_pieces), _stream()))
+        int(out_pieces), float(scale), _ptr(dyt_bias), _ptr(dyt_alpha), _stream()))
 
 
 @_op("scale_rows")

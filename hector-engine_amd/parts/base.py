@@ -215,9 +215,11 @@ class Part:
 
 
 class Norm(Part):
-    def carried(self) -> tuple[torch.Tensor, float] | None:
+    def carried(self) -> tuple | None:
         """(gain [D], eps) when the norm is y = x * gain / sqrt(mean(x^2) + eps), so that a
-        pair of products can carry it (ResidualSink, NormedRows); None otherwise."""
+        pair of products can carry it (ResidualSink, NormedRows); (gain [D], 1.0, bias [D], alpha)
+        when it is y = tanh(alpha x) * gain + bias, which the first product of the pair finishes
+        (the rows it leaves then owe nothing: sums of zero under eps 1); None otherwise."""
         return None
 
     def add_norm(self, resid: torch.Tensor, delta, rows: int, ctx: StepContext,
@@ -328,11 +330,13 @@ class ResidualSink:
     """Offered (ctx.sink) to a mixer or feed-forward whose output goes straight into the
     residual stream and then into `norm`: its last product may add its result to
     stream.resid itself and leave the rows for that norm (Linear(..., sink=ctx.take_sink())),
-    returning None instead of a tensor. A part that ignores the offer loses nothing."""
+    returning None instead of a tensor. A part that ignores the offer loses nothing. scale: the
+    stream gains scale * result."""
 
-    def __init__(self, stream: "ResidualStream", norm: Norm):
+    def __init__(self, stream: "ResidualStream", norm: Norm, scale: float = 1.0):
         self.stream = stream
         self.norm = norm
+        self.scale = scale
 
 
 class ResidualStream:
@@ -357,14 +361,15 @@ class ResidualStream:
         self.pending = delta
         self.pending_scale = scale
 
-    def sink_for(self, norm: Norm | None, ctx: StepContext) -> "ResidualSink | None":
+    def sink_for(self, norm: Norm | None, ctx: StepContext, scale: float = 1.0) -> "ResidualSink | None":
         """A sink for the part that runs next, when `norm` (the norm that will read the stream
-        after it) can be carried and the kernels for that are in use."""
+        after it) can be carried and the kernels for that are in use. scale: what the part's
+        result is multiplied by on its way into the stream."""
         if norm is None or self.pending is not None or norm.carried() is None:
             return None
         if not ctx.env.fast_kernels or ctx.env.dtype != torch.bfloat16:
             return None
-        return ResidualSink(self, norm)
+        return ResidualSink(self, norm, scale)
 
     def normed(self, norm: Norm, ctx: StepContext, rows_ok: bool = False):
         """norm(resid + pending) in the activation dtype. With rows_ok the caller takes

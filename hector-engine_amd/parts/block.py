@@ -49,16 +49,15 @@ class PreNormBlock(Block):
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
         after = ctx.next_norm                  # reads the stream once this block is done
         m = self.residual_scale
-        sinks = m == 1.0                       # a product that adds into the stream itself adds unscaled
         n = stream.normed(self.mixer_norm, ctx, self.mixer.accepts_normed_rows)
-        ctx.sink = stream.sink_for(self.ff_norm if self.feed_forward is not None else after, ctx) if sinks else None
+        ctx.sink = stream.sink_for(self.ff_norm if self.feed_forward is not None else after, ctx, m)
         delta = self.mixer.forward(n, ctx, cache)
         ctx.sink = None
         stream.add(delta, ctx, m)
         if self.feed_forward is None:
             return
         n = stream.normed(self.ff_norm, ctx, self.feed_forward.accepts_normed_rows)
-        ctx.sink = stream.sink_for(after, ctx) if sinks else None
+        ctx.sink = stream.sink_for(after, ctx, m)
         delta = self.feed_forward.forward(n, ctx)
         ctx.sink = None
         stream.add(delta, ctx, m)

@@ -249,27 +249,30 @@ class Linear:
         NormedRows: by the product's own epilogue, or, where it is cut along K, by the kernel
         that adds the slices."""
         N, K = self.weight.shape
-        gain, eps = sink.norm.carried()
+        gain, eps, *dyt = sink.norm.carried()
+        more = (sink.scale, *dyt) if dyt else (sink.scale,)      # (scale[, Dynamic Tanh's bias, alpha])
         out_pieces = N % 8 == 0
         xg = ctx.alloc(ops.pieces_shape(rows, N) if out_pieces else (rows, N), torch.bfloat16)
         _, a, scale, pieces = _operand(x)
         if rows <= ops.BLOCKSPLIT_PIECES_MAX_M:
             sq = ctx.alloc((rows, ops.gemm_blocksplit_blocks(rows, N, K)), torch.float32)
             ops.gemm_blocksplit(None, a, self.weight, bias, rows, row_scale=scale,
-                                residual=(sink.stream.resid, gain, xg, sq), x_pieces=pieces,
+                                residual=(sink.stream.resid, gain, xg, sq, *more), x_pieces=pieces,
                                 out_pieces=out_pieces)
         else:
             groups, splits = self._plan(rows)
             if splits == 1:
                 sq = ctx.alloc((rows, groups), torch.float32)
                 ops.gemm_rows(None, None, a, self.weight, bias, rows, row_scale=scale,
-                              residual=(sink.stream.resid, gain, xg, sq), x_pieces=pieces, out_pieces=out_pieces)
+                              residual=(sink.stream.resid, gain, xg, sq, *more), x_pieces=pieces,
+                              out_pieces=out_pieces)
             else:
                 partial = ctx.alloc((splits, rows, N), torch.float32)
                 ops.gemm_rows(None, partial, a, self.weight, None, rows, row_scale=scale, x_pieces=pieces)
                 sq = ctx.alloc((rows, ops.splitk_reduce_residual_blocks(N)), torch.float32)
                 ops.splitk_reduce_residual(sink.stream.resid, partial, bias, gain, xg, sq, rows, splits,
-                                           out_pieces=out_pieces)
+                                           out_pieces=out_pieces, scale=sink.scale,
+                                           dyt_bias=dyt[0] if dyt else None, dyt_alpha=dyt[1] if dyt else None)
         sink.stream.prepared = (sink.norm, NormedRows(xg, sq, eps, rows, out_pieces))
         return None
 

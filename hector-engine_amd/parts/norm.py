@@ -40,7 +40,8 @@ class RMSNorm(Norm):
 class DynamicTanh(Norm):
     """y = tanh(alpha * x) * weight + bias with a stored scalar alpha and vectors weight, bias: it
     stands where a norm would and computes neither a mean nor a variance, so no row is reduced and no
-    pair of products can carry it. Computed in fp32 on the fp32 residual stream, fused with the
+    pair of products has a row scale to carry; where a product adds into the stream itself (steps of
+    up to 64 rows), its epilogue computes this norm in full. Computed in fp32 on the fp32 residual stream, fused with the
     pending (scaled) residual add. names: suffixes of its tensors (weight, bias, alpha)."""
 
     def __init__(self, params: dict, prefix: str, env: BuildEnv):
@@ -61,6 +62,9 @@ class DynamicTanh(Norm):
         self.weight, self.bias, self.alpha = tensors[n["weight"]], tensors[n["bias"]], tensors[n["alpha"]]
         if not (self.weight.dtype == self.bias.dtype == self.alpha.dtype):
             raise TypeError(f"{self.prefix}: weight, bias and alpha are stored in different dtypes")
+
+    def carried(self):
+        return self.weight, 1.0, self.bias, self.alpha
 
     def add_norm(self, resid, delta, rows, ctx: StepContext, want_out: bool = True, delta_scale: float = 1.0):
         out = ctx.alloc((rows, self.size)) if want_out else None

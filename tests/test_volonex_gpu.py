@@ -65,6 +65,25 @@ def test_bounded_gated_activation(ops, dtype, rows, I, interleaved):
     assert (g.double() > 1.25).any() and (u.double() < -1.25).any()      # the bounds were met
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 20, 40, 64])
+@pytest.mark.parametrize("I,K", [(160, 264), (1008, 520)])
+def test_bounded_gated_activation_as_the_epilogue_of_a_product(ops, M, I, K):
+    x = rnd(M, K, seed=11).to(torch.bfloat16)
+    g, u = (rnd(I, K, seed=12) * 0.2).to(torch.bfloat16), (rnd(I, K, seed=13) * 0.2).to(torch.bfloat16)
+    w = torch.stack([g, u], 1).reshape(2 * I, K).contiguous()        # gate i at row 2i, its up at 2i + 1
+    out = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+    act = (1.702, 0.75, 1.0)
+    if M <= 16:
+        ops.gemm_blocksplit(out, dev(x), dev(w), None, M, gated=True, act=act)
+    else:
+        ops.gemm_rows(out, None, dev(x), dev(w), None, M, gated=True, plan=(0, 0, 1), act=act)
+    gd = (x.double() @ g.double().T).clamp(max=0.75)
+    ud = (x.double() @ u.double().T).clamp(-0.75, 0.75)
+    assert (x.double() @ g.double().T > 0.75).any()
+    want = gd * torch.sigmoid(1.702 * gd) * (ud + 1)
+    assert torch.allclose(out.cpu().double(), want, rtol=2 ** -7, atol=2 ** -7)
+
+
 def test_embedding_scale_and_scaled_residual_add(ops):
     table = rnd(50, 24, seed=7).to(torch.bfloat16)
     ids = torch.tensor([3, 49, 0, 7], dtype=torch.int32)
