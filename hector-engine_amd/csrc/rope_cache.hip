@@ -127,8 +127,9 @@ __global__ void qkv_rope_cache_kernel(
 }
 
 // bf16 rows, eight elements per access: one thread rotates the pairs (j..j+7, j+half..)
-// of one head, or copies eight v elements. Needs rotary_dim/2, head_dim - rotary_dim and
-// the row stride in multiples of 8.
+// of one head (interleaved: the four pairs inside eight neighbouring dims), or copies eight v
+// elements. Needs rotary_dim/2 (interleaved: rotary_dim), the head sizes, head_dim - rotary_dim and
+// the row stride in multiples of 8. hd_in, vd_in, interleaved, mscale: as the kernel above takes them.
 __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -145,7 +146,7 @@ __device__ __forceinline__ uint4 pack8(const float* f) {
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// grid: one workgroup per 8 rows for v, then one per row for q and k.
+// grid: one workgroup per 8 rows (per row in a step of up to 128 rows) for v, then one per row for q and k.
 // V lies transposed in a page (8 keys of one dim are 16 contiguous bytes), so the v values of
 // a run of tokens that share such a group are gathered dim by dim and stored together: 16
 // bytes a store when the run is a whole group (a prompt), 2 bytes a token otherwise.
@@ -157,14 +158,16 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
     int num_pages, const float* __restrict__ inv_freq, int rotary_dim, int rows, int H, int KVH,
-    int hd) {
+    int hd, int hd_in, int vd_in, int interleaved, float mscale, int v_span) {
   __shared__ float cs[2][ROPE_MAX_HALF];
   const int v_blocks = (int)gridDim.x - rows;   // they come first: theirs is the longest chain of dependent loads
   if ((int)blockIdx.x < v_blocks) {
-    // ---- v: the runs of tokens that begin in rows [r0, r0 + 8)
-    const int r0 = 8 * (int)blockIdx.x;
+    // ---- v: the runs of tokens that begin in rows [r0, r0 + v_span). In a step of few rows (one token a
+    // sequence) every row has a workgroup of its own: a workgroup takes its rows one after the other, and
+    // each is a chain of dependent loads (sequence, slot, page) that eight rows in a row made 14 us long.
+    const int r0 = v_span * (int)blockIdx.x;
     const int NT = he_v_tiles(hd);
-    for (int r = r0; r < min(r0 + 8, rows); ++r) {
+    for (int r = r0; r < min(r0 + v_span, rows); ++r) {
       const int seq = row_seq[r];
       if (seq < 0) continue;
       const int pos = positions[r];
@@ -175,8 +178,8 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
       const int page = page_table[(int64_t)seq_slot[seq] * max_blocks + (pos >> HE_PAGE_SHIFT)];
       if (page < 0 || page >= num_pages) continue;
       const int off = pos & (HE_PAGE_TOKENS - 1);
-      for (int e = threadIdx.x; e < KVH * hd; e += blockDim.x) {
-        const int h = e / hd, d = e - h * hd;
+      for (int e = threadIdx.x; e < KVH * vd_in; e += blockDim.x) {
+        const int h = e / vd_in, d = e - h * vd_in;
         const float b = v_bias ? bf16_bits_to_float(v_bias[e]) : 0.f;
         uint16_t vals[8];
         // eight loads with no branch around them (a token beyond the run reads the run's last
@@ -207,44 +210,48 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
   const int seq = row_seq[row];
   if (seq < 0) return;  // padding row
   const int half = rotary_dim >> 1;
-  const int rot8 = half >> 3;                 // groups of 8 pairs per head
-  const int pass8 = (hd - rotary_dim) >> 3;   // groups of 8 pass-through dims per head
-  const int per_head = rot8 + pass8;
-  const int q_items = H * per_head;
-  const int items = q_items + (k_in ? KVH * per_head : 0);
-  // an item: eight pairs (j.., j + half..) of one head, or eight pass-through dims from d on
+  const int rot8 = (interleaved ? rotary_dim : half) >> 3;   // rotated groups per head: 8 pairs, or, interleaved, 8 dims
+  // groups of 8 pass-through dims per head: q_out has hd dims a head (those from hd_in on are zeros), a key hd_in
+  const int per_head_q = rot8 + ((hd - rotary_dim) >> 3), per_head_k = rot8 + ((hd_in - rotary_dim) >> 3);
+  const int q_items = H * per_head_q;
+  const int items = q_items + (k_in ? KVH * per_head_k : 0);
+  // an item: eight pairs (j.., j + half..) of one head (interleaved: the dims j..j+7, four pairs), or eight
+  // pass-through dims from j on
   struct Item {
     const uint16_t* in;
     const uint16_t* bias;
     int h, j;
-    bool is_q, rotated;
+    bool is_q, rotated, pad;
   };
   auto item = [&](int it) {
     Item im;
     im.is_q = it < q_items;
     const int idx = im.is_q ? it : it - q_items;
+    const int per_head = im.is_q ? per_head_q : per_head_k;
     im.h = idx / per_head;
     const int g = idx - im.h * per_head;
     im.rotated = g < rot8;
     im.j = im.rotated ? 8 * g : rotary_dim + 8 * (g - rot8);
-    im.in = (im.is_q ? q_in : k_in) + row * in_stride + im.h * hd;
+    im.pad = !im.rotated && im.j >= hd_in;       // dims of q_out beyond the rows' head size
+    im.in = (im.is_q ? q_in : k_in) + row * in_stride + im.h * hd_in;
     const uint16_t* bias = im.is_q ? q_bias : k_bias;
-    im.bias = bias ? bias + im.h * hd : nullptr;
+    im.bias = bias ? bias + im.h * hd_in : nullptr;
     return im;
   };
   const uint4 zero = make_uint4(0, 0, 0, 0);
   // four loads with no branch around them, so that they go out together: an item without a
   // partner, or a row without a bias, reads its own eight elements again and drops them
   auto load = [&](const Item& im, uint4 (&raw)[4]) {
-    const int partner = im.rotated ? im.j + half : im.j;
+    const int j = im.pad ? 0 : im.j;             // (padding reads the head's first dims and drops them)
+    const int partner = im.rotated && !interleaved ? j + half : j;
     const uint16_t* b = im.bias ? im.bias : im.in;
-    const uint4 x0 = *reinterpret_cast<const uint4*>(im.in + im.j);
+    const uint4 x0 = *reinterpret_cast<const uint4*>(im.in + j);
     const uint4 x1 = *reinterpret_cast<const uint4*>(im.in + partner);
-    const uint4 b0 = *reinterpret_cast<const uint4*>(b + im.j);
+    const uint4 b0 = *reinterpret_cast<const uint4*>(b + j);
     const uint4 b1 = *reinterpret_cast<const uint4*>(b + partner);
-    raw[0] = x0;
+    raw[0] = im.pad ? zero : x0;
     raw[1] = im.rotated ? x1 : zero;
-    raw[2] = im.bias ? b0 : zero;
+    raw[2] = im.bias && !im.pad ? b0 : zero;
     raw[3] = im.bias && im.rotated ? b1 : zero;
   };
   // the loads of a thread's first item are on their way while the angles are computed
@@ -261,8 +268,8 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     float sn, c;
     sincos_angle((float)pos * inv_freq[i], &sn, &c);
-    cs[0][i] = c;
-    cs[1][i] = sn;
+    cs[0][i] = c * mscale;
+    cs[1][i] = sn * mscale;
   }
   __syncthreads();
   const bool cache_ok = page >= 0 && page < num_pages;
@@ -281,7 +288,17 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
     float x0[8], x1[8], b0[8], b1[8];
     unpack8(raw[0], x0);
     unpack8(raw[2], b0);
-    if (im.rotated) {
+    if (im.rotated && interleaved) {
+      float y[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float a0 = x0[2 * i] + b0[2 * i], a1 = x0[2 * i + 1] + b0[2 * i + 1];
+        const float c = cs[0][(im.j >> 1) + i], sn = cs[1][(im.j >> 1) + i];
+        y[2 * i] = a0 * c - a1 * sn;
+        y[2 * i + 1] = a0 * sn + a1 * c;
+      }
+      *reinterpret_cast<uint4*>(at(im.j)) = pack8(y);
+    } else if (im.rotated) {
       unpack8(raw[1], x1);
       unpack8(raw[3], b1);
       float y0[8], y1[8];
@@ -346,23 +363,25 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
       (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot,             \
       (const int32_t*)page_table, max_blocks, num_pages, (const float*)inv_freq, rotary_dim, H, \
       KVH, hd, hd_in, vd_in, interleaved, mscale)
-  const bool vec_ok = dtype == HE_BF16 && hd_in == hd && vd_in == hd && !interleaved && mscale == 1.f &&
+  const bool vec_ok = dtype == HE_BF16 &&
                       (q_bias == nullptr || bias_dtype == HE_BF16) &&
-                      ((rotary_dim >> 1) & 7) == 0 && ((hd - rotary_dim) & 7) == 0 &&
-                      (in_stride & 7) == 0 && (hd & 7) == 0 &&
+                      ((interleaved ? rotary_dim : rotary_dim >> 1) & 7) == 0 && ((hd - rotary_dim) & 7) == 0 &&
+                      (in_stride & 7) == 0 && (hd & 7) == 0 && (hd_in & 7) == 0 &&
                       ((((uintptr_t)q_in) | ((uintptr_t)k_in) | ((uintptr_t)v_in) |
                         ((uintptr_t)q_bias) | ((uintptr_t)k_bias) | ((uintptr_t)v_bias) |
                         ((uintptr_t)q_out) | ((uintptr_t)kpool)) & 15) == 0;
   if (vec_ok) {
-    const int items = (H + (k_in ? KVH : 0)) * ((rotary_dim >> 4) + ((hd - rotary_dim) >> 3));
+    const int rot8 = (interleaved ? rotary_dim : rotary_dim >> 1) >> 3;
+    const int items = H * (rot8 + ((hd - rotary_dim) >> 3)) + (k_in ? KVH * (rot8 + ((hd_in - rotary_dim) >> 3)) : 0);
     const int vec_threads = min(1024, max(64, (items + 63) / 64 * 64));
-    const int v_blocks = k_in ? (rows + 7) / 8 : 0;
+    const int v_span = rows <= 128 ? 1 : 8;
+    const int v_blocks = k_in ? (rows + v_span - 1) / v_span : 0;
     qkv_rope_cache_vec_kernel<<<rows + v_blocks, vec_threads, 0, s>>>(
         (uint16_t*)q_out, (uint16_t*)kpool, (uint16_t*)vpool, (const uint16_t*)q_in,
         (const uint16_t*)k_in, (const uint16_t*)v_in, in_stride, (const uint16_t*)q_bias,
         (const uint16_t*)k_bias, (const uint16_t*)v_bias, (const int32_t*)positions,
         (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,
-        num_pages, (const float*)inv_freq, rotary_dim, rows, H, KVH, hd);
+        num_pages, (const float*)inv_freq, rotary_dim, rows, H, KVH, hd, hd_in, vd_in, interleaved, mscale, v_span);
   } else if (dtype == HE_BF16) {
     ROPE_LAUNCH(bf16_t, bf16_t);
   } else {

@@ -137,6 +137,9 @@ class Attention(Mixer):
         gate_w = tensors.pop(n["gate"]) if self.head_gate else None
         if gate_w is not None:
             ws.append(gate_w)          # the gate's rows ride behind q||k||v: one product
+            spare = -sum(w.shape[0] for w in ws) % 8
+            if spare:                  # rows of zeros, so that the product's rows stay a multiple of 8 wide
+                ws.append(torch.zeros((spare, gate_w.shape[1]), dtype=gate_w.dtype, device=gate_w.device))
         if len({w.dtype for w in ws}) != 1:
             raise TypeError(f"{p}q/k/v projections are stored in different dtypes")
         w = torch.cat(ws, 0).contiguous() if len(ws) > 1 else ws[0]
@@ -146,13 +149,22 @@ class Attention(Mixer):
             if len({x.dtype for x in bs}) != 1:
                 raise TypeError(f"{p}q/k/v biases are stored in different dtypes")
             b = torch.cat(bs, 0).contiguous() if len(bs) > 1 else bs[0]
-        self.qkv = Linear(w, b)
+        def bias_for(bias, rows):
+            """The bias, with zeros for the rows behind q||k||v (the gates and the spare rows)."""
+            if bias is None or bias.numel() == rows:
+                return bias
+            return torch.cat([bias, torch.zeros(rows - bias.numel(), dtype=bias.dtype, device=bias.device)])
+
+        self.qkv = Linear(w, bias_for(b, w.shape[0]))
         q_rows = self.H * self.hd
         if gate_w is not None and self.kv_projection:
-            self.q_only = Linear(torch.cat([ws[0], gate_w], 0).contiguous(), None if b is None else b[:q_rows])
+            spare = -(q_rows + self.H) % 8
+            self.q_only = Linear(torch.cat([ws[0], gate_w, torch.zeros((spare, gate_w.shape[1]), dtype=gate_w.dtype,
+                                                                       device=gate_w.device)], 0).contiguous(),
+                                 None if b is None else bias_for(b[:q_rows], q_rows + self.H + spare))
         else:
-            self.q_only = Linear(w[:q_rows + (self.H if gate_w is not None else 0)],
-                                 None if b is None else b[:q_rows])
+            self.q_only = Linear(w if gate_w is not None else w[:q_rows],
+                                 None if b is None else bias_for(b[:q_rows], w.shape[0] if gate_w is not None else q_rows))
         del ws
         wo = tensors[n["o"]]
         if self.pd != self.vd:

@@ -560,3 +560,39 @@ def test_greedy_generation_through_the_library(folders, plain, name):
                 assert (top[0] - top[1]).item() < 0.03 * top[0].abs().item() + 1e-3      # a near tie
                 break
             seq.append(x)
+
+
+def test_the_command_line_and_the_trace_replay_serve_it(folders, plain, tmp_path):
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from tests.conftest import ROOT
+    cfg, w = plain["V1"]
+    exe = os.path.join(ROOT, "bin", "hector_generate")
+    out = subprocess.run([sys.executable, exe, folders["V1"], "5,17,3;9,2,77,13", "6", "--dtype", "float32",
+                          "--stop-ids", ""], capture_output=True, text=True, timeout=180)
+    assert out.returncode == 0, out.stderr
+    for i, p in enumerate(([5, 17, 3], [9, 2, 77, 13])):
+        assert f"[{i}] prompt" in out.stdout and ",".join(map(str, P.greedy(cfg, w, p, 6))) in out.stdout
+    assert "Volonex" in out.stdout
+    # a replay whose requests need more pages than their token count alone suggests (each request's
+    # last page is partly empty): 196 tokens live at once, in 1 + 2 + 3 pages
+    reqs = {"a": rand_ids(cfg["vocab"], 4, 1), "b": rand_ids(cfg["vocab"], 68, 2), "c": rand_ids(cfg["vocab"], 133, 3)}
+    steps = [{"step": 0, "entries": [{"id": k, "tokens": v[:-3], "want": [len(v) - 4]} for k, v in reqs.items()], "end": []}]
+    for t in range(3):
+        steps.append({"step": t + 1, "entries": [{"id": k, "tokens": [v[len(v) - 3 + t]], "want": [0]} for k, v in reqs.items()],
+                      "end": list(reqs) if t == 2 else []})
+    for dtype in DTYPES:
+        out_dir = str(tmp_path / dtype)
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders["V1"],
+                               "--dtype", dtype, "--out", out_dir, "--max-tokens", "196"],
+                              input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=180)
+        assert proc.returncode == 0, proc.stderr
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+        want = {k: P.forward(cfg, w, v) for k, v in reqs.items()}
+        for s in range(4):
+            got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{s}.f32"), dtype="<f4").reshape(3, -1).copy())
+            rows = torch.stack([want[k][len(reqs[k]) - 4 + s] for k in reqs])
+            close(got, rows, dtype)
