@@ -115,14 +115,14 @@ def attention(h, positions, mx: dict, w: dict, prefix: str, k_cache=None, v_cach
         v_cache[:] = vals
     chunk = (mx.get("mask") or {}).get("size", 0)
     out = torch.zeros(T, H, e, dtype=F64)
+    all_k, all_v = torch.stack(keys), torch.stack(vals)        # [n, G, d], [n, G, e]
     for t, p in enumerate(positions):
         js = [n for n, pj in enumerate(where) if sees(p, pj, chunk)]
         for head in range(H):
             kv = head // (H // G)
-            s = torch.stack([(q[t, head] * keys[n][kv]).sum() for n in js]) * mx["scale"]
+            s = (all_k[js, kv] @ q[t, head]) * mx["scale"]       # one score a visible key
             a = softmax_with_sink(s, w[prefix + "sink"][head])
-            o = sum(a[x] * vals[n][kv] for x, n in enumerate(js))
-            out[t, head] = o * gate[t, head]
+            out[t, head] = (a @ all_v[js, kv]) * gate[t, head]
     return out.reshape(T, H * e) @ w[prefix + "o"].T
 
 

@@ -166,10 +166,9 @@ def plain_attention(q, k, v, q_pos, chunk, window, scale, sinks, gate):
         js = [j for j in range(k.shape[0]) if P.sees(p, j, chunk, window)]
         for h in range(H):
             kv = h // (H // G)
-            s = torch.stack([(q[t, h] * k[j, kv]).sum() for j in js]) * scale
+            s = (k[js, kv] @ q[t, h]) * scale
             a = P.softmax_with_sink(s, sinks[h]) if sinks is not None else torch.softmax(s, 0)
-            o = sum(a[x] * v[j, kv] for x, j in enumerate(js))
-            out[t, h] = o * (torch.sigmoid(gate[t, h]) if gate is not None else 1.0)
+            out[t, h] = (a @ v[js, kv]) * (torch.sigmoid(gate[t, h]) if gate is not None else 1.0)
     return out
 
 
