@@ -83,7 +83,7 @@ class PagedCache:
         self.groups = [_Group(k, m, self.num_pages, self.max_slots, self.max_blocks, dtype, device)
                        for k, m in zip(keys, members)]
         self.book = SlotBook(self.max_slots, self.max_blocks,
-                             [GroupPages(self.num_pages, k.window, f"{i}") for i, k in enumerate(keys)])
+                             [GroupPages(self.num_pages, k.window, f"{i}", k.chunk) for i, k in enumerate(keys)])
 
         # fixed-size per-sequence state: one row per slot, one span per run
         self.state_offsets: list[int] = []

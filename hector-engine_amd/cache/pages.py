@@ -57,10 +57,12 @@ def blocks_for(length: int) -> int:
 
 
 class GroupPages:
-    """Pages of one group of layers: all keys (window 0) or the last `window`."""
+    """Pages of one group of layers: all keys (window 0) or the last `window`; with chunk > 0 a
+    query reads no key before the start of its own chunk of that many positions."""
 
-    def __init__(self, num_pages: int, window: int, name: str):
+    def __init__(self, num_pages: int, window: int, name: str, chunk: int = 0):
         self.window = window
+        self.chunk = chunk
         self.pool = FreeList(num_pages, f"page of cache group {name}")
         # slot -> list over blocks of a page id, or -1 once the block left the window
         self.table: dict[int, list[int]] = {}
@@ -132,17 +134,18 @@ class SlotBook:
         return added
 
     def commit(self, slot: int, new_length: int) -> list[tuple[int, int, int]]:
-        """Records the new length and gives back the pages of windowed groups
+        """Records the new length and gives back the pages of windowed and chunked groups
         that no later query can see: block b is dead once its last position
-        64b+63 <= new_length - window. Returns cleared (group, slot, block)."""
+        64b+63 <= new_length - window, or lies before the chunk that position new_length is in.
+        Returns cleared (group, slot, block)."""
         self._check(slot)
         self.length[slot] = new_length
         cleared = []
         for gi, g in enumerate(self.groups):
-            if g.window <= 0:
+            if g.window <= 0 and g.chunk <= 0:
                 continue
             row = g.table[slot]
-            for b in range(min(self._dead_blocks(new_length, g.window), len(row))):
+            for b in range(min(self._dead_blocks(new_length, g.window, g.chunk), len(row))):
                 if row[b] >= 0:
                     g.pool.give_back(row[b])
                     row[b] = -1
@@ -161,11 +164,12 @@ class SlotBook:
         if not 0 <= new_length <= self.length[slot]:
             raise CacheError(f"slot {slot}: cannot truncate from {self.length[slot]} to {new_length}")
         for gi, g in enumerate(self.groups):
-            if g.window <= 0:
+            if g.window <= 0 and g.chunk <= 0:
                 continue
-            dead = self._dead_blocks(new_length, g.window)
+            dead = self._dead_blocks(new_length, g.window, g.chunk)
             if any(page < 0 for page in g.table[slot][dead:]):
-                raise CacheError(f"slot {slot}: group {gi} keeps a window of {g.window} keys and has given "
+                kept = f"a window of {g.window} keys" if g.window > 0 else f"the keys of a chunk of {g.chunk}"
+                raise CacheError(f"slot {slot}: group {gi} keeps {kept} and has given "
                                  f"back pages that a sequence of {new_length} tokens still reads")
         keep = blocks_for(new_length)
         cleared = []
@@ -180,12 +184,16 @@ class SlotBook:
         return cleared
 
     @staticmethod
-    def _dead_blocks(length: int, window: int) -> int:
-        """Leading blocks of a windowed group that no query at or beyond position `length`
-        reads: block b is dead once its last position 64b+63 <= length - window."""
-        if length - window < PAGE_TOKENS - 1:
-            return 0
-        return (length - window - (PAGE_TOKENS - 1)) // PAGE_TOKENS + 1
+    def _dead_blocks(length: int, window: int, chunk: int = 0) -> int:
+        """Leading blocks that no query at or beyond position `length` reads: block b is dead
+        once its last position 64b+63 <= length - window (a window), or < the first position of
+        the chunk that `length` lies in (chunks: a later query's chunk starts there or later)."""
+        dead = 0
+        if window > 0 and length - window >= PAGE_TOKENS - 1:
+            dead = (length - window - (PAGE_TOKENS - 1)) // PAGE_TOKENS + 1
+        if chunk > 0:
+            dead = max(dead, (length - length % chunk) // PAGE_TOKENS)
+        return dead
 
     def check_invariants(self) -> None:
         """Every page is free or held by exactly one (slot, block)."""

@@ -72,7 +72,7 @@ class Session:
         # Step by step where a queued step could not be taken back: a stop token read late has been
         # fed by the step queued behind it, and a group that keeps a window may have given a page away
         # by then.
-        windowed = any(g.window > 0 for g in engine.cache.book.groups)
+        windowed = any(g.window > 0 or g.chunk > 0 for g in engine.cache.book.groups)
         stepwise = run_of_steps <= 1 or (config.has_penalties and not getattr(sampler, "window_on_device", False)) \
             or (windowed and bool(self.stop_ids))
         results: list[GenerationResult | None] = [None]

@@ -107,7 +107,7 @@ class Attention(Mixer):
     def kv_need(self):
         # pages in the order the attention kernels read their operands
         return KVNeed(self.KVH, self.pd, self.window, k_page_elems=kv_layout.k_page_elems(self.pd),
-                      v_page_elems=kv_layout.v_page_elems(self.pd))
+                      v_page_elems=kv_layout.v_page_elems(self.pd), chunk=self.chunk)
 
     def tensor_specs(self):
         n, hd, vd = self._names, self.hd, self.vd

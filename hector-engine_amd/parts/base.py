@@ -85,7 +85,9 @@ PAGE_TOKENS = 64     # tokens of a cache page
 class KVNeed:
     """What a mixer keeps per token in the cache: per kv head a key of `head_dim` and a value
     of `value_dim` elements (0: as wide as the key), all of them (window 0) or only the last
-    `window`. Mixers with equal needs share a group of the cache.
+    `window`; with `chunk` > 0 nothing before the start of the chunk of that many positions that the
+    newest position lies in (the cache gives back the pages before it). Mixers with equal needs
+    share a group of the cache.
 
     k_page_elems, v_page_elems: the elements of one page (64 tokens of one kv head) in the
     group's two pools. The order inside a page is the mixer's own business: the cache hands out
@@ -100,6 +102,7 @@ class KVNeed:
     value_dim: int = 0
     k_page_elems: int = 0
     v_page_elems: int = 0
+    chunk: int = 0
 
     @property
     def v_dim(self) -> int:

@@ -249,3 +249,30 @@ def test_the_host_copy_of_the_page_tables_follows_the_device_tables():
             pass
         check()
     assert any((g.host_table >= 0).any() for g in cache.groups)
+
+
+@pytest.mark.parametrize("chunk", [1, 24, 64, 70, 200])
+def test_chunked_group_frees_the_blocks_before_the_running_chunk(chunk):
+    b = SlotBook(4, 16, [GroupPages(32, 0, "all"), GroupPages(32, 0, "chunked", chunk)])
+    s = b.acquire()
+    length = 0
+    for grow in [1, 23, 40, 1, 63, 64, 65, 1, 1, 130, 200]:
+        length += grow
+        b.reserve(s, length)
+        b.commit(s, length)
+        start = length - length % chunk          # the next query (position `length`) sees nothing before this
+        row = b.groups[1].table[s]
+        for blk, page in enumerate(row):
+            dead = 64 * blk + 63 < start
+            assert (page < 0) == dead, (length, blk)
+        assert all(page >= 0 for page in b.groups[0].table[s])
+        b.check_invariants()
+    # a cut back into a chunk whose pages are gone is refused and changes nothing
+    if chunk >= 64:
+        with pytest.raises(CacheError, match="chunk"):
+            b.truncate(s, 1)
+        assert b.length[s] == length
+    b.truncate(s, length - length % chunk)       # the start of the running chunk still has its keys' pages ahead of it
+    b.check_invariants()
+    b.release(s)
+    assert all(g.pool.available == 32 for g in b.groups)

@@ -595,3 +595,18 @@ def test_the_command_line_and_the_trace_replay_serve_it(folders, plain, tmp_path
             got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{s}.f32"), dtype="<f4").reshape(3, -1).copy())
             rows = torch.stack([want[k][len(reqs[k]) - 4 + s] for k in reqs])
             close(got, rows, dtype)
+
+
+def test_pages_before_the_running_chunk_go_back_to_the_pool(engines, plain):
+    eng = engines("V2", "float32")
+    cfg, w = plain["V2"]
+    ids = rand_ids(cfg["vocab"], 300, 5)
+    free = eng.cache.free_pages
+    s = eng.acquire()
+    eng.step([entry(s, ids[:290], [])])
+    got = torch.cat([eng.step([entry(s, [t], [0])]).clone() for t in ids[290:]])
+    close(got, P.forward(cfg, w, ids)[290:], "float32")
+    held = {g.chunk: sum(p >= 0 for p in g.table[s]) for g in eng.cache.book.groups}
+    assert held == {16: 1, 0: 5, 128: 1}          # 300 tokens lie in five pages; the chunks that run began at 288 and 256
+    eng.release(s)
+    assert eng.cache.free_pages == free
