@@ -1,4 +1,5 @@
-"""Qwen2 dense generation library for one MI355X (package folder ``hector-engine_amd``).
+"""Generation library for one MI355X (package folder ``hector-engine_amd``): Qwen2 dense decoders and
+the Volonex design, both assembled from the same registered parts.
 
 Python entry point:
 
