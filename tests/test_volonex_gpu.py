@@ -299,6 +299,27 @@ def test_a_planted_key_at_the_edge_of_a_chunk(ops, kind, where):
     assert seen == (where != "just_outside")
 
 
+@pytest.mark.parametrize("kind", ["plain32", "plain", "decode", "prefill"])
+@pytest.mark.parametrize("at", [3, 63, 64, 640])
+@pytest.mark.parametrize("chunk", [0, 1024])
+def test_a_planted_key_far_back_among_hundreds(ops, kind, at, chunk):
+    """The last query's answer lies hundreds of keys back (near the start, on either side of a page
+    border, ten pages in): a kernel that drops a slice, a part or a page of the keys loses it."""
+    dtype = torch.float32 if kind == "plain32" else torch.bfloat16
+    H, KVH, hd, n = 6, 3, 48, 900
+
+    def plant(qs, ks, vs):
+        direction = torch.ones(hd) / math.sqrt(hd)
+        qs[0][-1] = (direction * 40).to(dtype)
+        ks[0][at] = (direction * 40).to(dtype)
+        vs[0][at] = torch.full((KVH, hd), 25.0).to(dtype)
+
+    q_lens = [1] if kind == "decode" else [n] if kind == "prefill" else [2]
+    got, want = run_attention(ops, kind.replace("32", ""), dtype, H, KVH, hd, chunk, 0, [n], q_lens, 95, plant=plant)
+    same(got, want, dtype)
+    assert want[0][-1].abs().max().item() > 5
+
+
 @pytest.mark.parametrize("kind", ["plain", "decode", "prefill"])
 def test_a_large_sink_takes_the_weight_away(ops, kind):
     """A sink far above every score leaves almost nothing for the keys: a kernel that forgot it
