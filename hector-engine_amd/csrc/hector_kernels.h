@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 21
+#define HE_ABI_VERSION 22
 
 #ifdef __cplusplus
 extern "C" {
@@ -133,11 +133,12 @@ int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in, c
                       const void* row_seq, const void* seq_slot, const void* page_table,
                       int max_blocks, int num_pages, const void* inv_freq, int rotary_dim, int rows,
                       int H, int KVH, int hd, int hd_in, int vd_in, int interleaved, float mscale,
-                      int dtype, void* stream);
+                      float q_coef, int q_every, int dtype, void* stream);
 // hd: head size of q_out and of the cache pages. hd_in, vd_in (0: hd): head sizes of the q/k rows and
 // of the v rows that come in (at most hd; q_out is padded with zeros, the pages keep their zeros).
 // interleaved: frequency i turns the pair (2i, 2i + 1), not (i, i + rotary_dim / 2). mscale multiplies
-// cos and sin.
+// cos and sin. q_every > 0: the q of a row at position p is multiplied by
+// 1 + q_coef * ln(floor((p + 1) / q_every) + 1) (a query temperature that grows with the position).
 
 // ---- attention over the paged cache ----------------------------------------
 // he_attention_plain: fp32 sums in one fixed order per (query, head): page by page (64 positions),
@@ -207,6 +208,36 @@ int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const
                               int kernel, int total_rows, int parts, void* workspace_f32,
                               int64_t workspace_floats, int chunk, const void* sinks, int sinks_dtype,
                               const void* gate, int64_t gate_stride, void* stream);
+
+// ---- state-space mixer (state_space.hip) ------------------------------------
+// A sequence's row of the state area holds, in fp32, the last K-1 inputs of the convolution [K-1][C] at
+// its start, and the scan's state at state_offset, he_ssm_state_floats(R, P, N) floats.
+// out[row, c] = silu(bias[c] + sum_j taps[c][j] * x[row - (K-1) + j, c]) within a sequence (inputs before the
+// step come from the carried ones), then the carried inputs move on. x: [rows][>= C] at x_stride elements.
+int he_conv_state(void* out, const void* x, int64_t x_stride, const void* taps, const void* bias,
+                  int w_dtype, void* state, int64_t state_stride, const void* positions,
+                  const void* row_seq, const void* seq_slot, const void* seq_start,
+                  const void* cu_seqlens, int rows, int num_seqs, int C, int K, int all_single,
+                  int dtype, void* stream);
+int64_t he_ssm_state_floats(int R, int P, int N);
+// xbc [rows][R P + 2 Q N]: x, then the Q groups' B vectors, then their C vectors; dt_in[row * dt_stride + r].
+// y [rows][R P] fp32 (rows without a sequence are not written).
+int he_ssm_scan(void* y_f32, const void* xbc, const void* dt_in, int64_t dt_stride, const void* dt_bias,
+                const void* a_log, const void* d_skip, int w_dtype, void* state, int64_t state_stride,
+                int64_t state_offset, const void* cu_seqlens, const void* seq_slot, int rows, int num_seqs,
+                int R, int Q, int N, int P, int dtype, void* stream);
+// out = rms over each of `parts` stretches of (y * silu(z)) * weight; z[row * z_stride + c].
+int he_gated_group_norm(void* out, const void* y_f32, const void* z, int64_t z_stride, const void* weight,
+                        int w_dtype, int rows, int W, int parts, float eps, int dtype, void* stream);
+
+// ---- routing and head combination (routing.hip) ---------------------------------
+int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32, const void* logits_f32,
+                    const void* correction, int c_dtype, int rows, int E, int real, int groups, int keep,
+                    int top, float scale, void* stream);
+int he_routed_act(void* out, const void* gate_up, const void* dense_f32, const void* h, int rows, int real,
+                  int I, int extra, int dtype, float alpha, float limit, float up_shift, void* stream);
+int he_diff_heads(void* out, const void* attn, int rows, int H, int G, int hd, int vd, float lambda,
+                  float post, float eps, int dtype, void* stream);
 
 // ---- sampling ------------------------------------------------------------
 int64_t he_argmax_workspace_bytes(int rows, int V);

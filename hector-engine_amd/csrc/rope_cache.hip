@@ -13,6 +13,12 @@
 
 #define ROPE_MAX_HALF 256
 
+// A query's temperature: q at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1), so
+// that queries far into a sequence are sharper (every <= 0: none). In fp32.
+__device__ __forceinline__ float he_query_temperature(int pos, float coef, int every) {
+  return every > 0 ? fmaf(coef, logf((float)((pos + 1) / every + 1)), 1.f) : 1.f;
+}
+
 // hd: the head size of q_out and of the cache pages; hd_in <= hd, vd_in <= hd: the head sizes of the
 // projected q/k and v rows (a mixer whose keys and values differ in width keeps both in pages of
 // the wider one: q_out's dims from hd_in on are written as zeros, those of the pages are never
@@ -27,12 +33,13 @@ __global__ void qkv_rope_cache_kernel(
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ page_table, int max_blocks, int num_pages,
     const float* __restrict__ inv_freq, int rotary_dim, int H, int KVH, int hd, int hd_in, int vd_in,
-    int interleaved, float mscale) {
+    int interleaved, float mscale, float q_coef, int q_every) {
   __shared__ float cs[2][ROPE_MAX_HALF];
   const int64_t row = blockIdx.x;
   const int seq = row_seq[row];
   if (seq < 0) return;  // padding row
   const int pos = positions[row];
+  const float q_mul = he_query_temperature(pos, q_coef, q_every);
   const int half = rotary_dim >> 1;
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const float a = (float)pos * inv_freq[i];
@@ -64,8 +71,8 @@ __global__ void qkv_rope_cache_kernel(
           x1 += load_param(q_bias, base + d1, bias_dtype);
         }
         const float c = cs[0][j], sn = cs[1][j];
-        out[obase + d0] = from_float<T>(x0 * c - x1 * sn);
-        out[obase + d1] = from_float<T>(x0 * sn + x1 * c);
+        out[obase + d0] = from_float<T>((x0 * c - x1 * sn) * q_mul);
+        out[obase + d1] = from_float<T>((x0 * sn + x1 * c) * q_mul);
       } else {
         const int d = rotary_dim + (j - half);
         float x = 0.f;
@@ -73,7 +80,7 @@ __global__ void qkv_rope_cache_kernel(
           x = to_float((in + base + d)[0]);
           if (q_bias) x += load_param(q_bias, base + d, bias_dtype);
         }
-        out[obase + d] = from_float<T>(x);
+        out[obase + d] = from_float<T>(x * q_mul);
       }
     }
   }
@@ -158,7 +165,7 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
     int num_pages, const float* __restrict__ inv_freq, int rotary_dim, int rows, int H, int KVH,
-    int hd, int hd_in, int vd_in, int interleaved, float mscale, int v_span) {
+    int hd, int hd_in, int vd_in, int interleaved, float mscale, int v_span, float q_coef, int q_every) {
   __shared__ float cs[2][ROPE_MAX_HALF];
   const int v_blocks = (int)gridDim.x - rows;   // they come first: theirs is the longest chain of dependent loads
   if ((int)blockIdx.x < v_blocks) {
@@ -275,6 +282,8 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
   const bool cache_ok = page >= 0 && page < num_pages;
   const int off = pos & (HE_PAGE_TOKENS - 1);
   const int KS = he_k_steps(hd);
+  const float q_mul = he_query_temperature(pos, q_coef, q_every);
+  const bool tempered = q_mul != 1.f;
   auto finish = [&](const Item& im, const uint4 (&raw)[4]) {
     // where the eight elements from dim d on go: the q row, or the cache page in operand order
     uint16_t* out;
@@ -297,6 +306,10 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
         y[2 * i] = a0 * c - a1 * sn;
         y[2 * i + 1] = a0 * sn + a1 * c;
       }
+      if (im.is_q && tempered) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] *= q_mul;
+      }
       *reinterpret_cast<uint4*>(at(im.j)) = pack8(y);
     } else if (im.rotated) {
       unpack8(raw[1], x1);
@@ -309,12 +322,20 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
         y0[i] = a0 * c - a1 * sn;
         y1[i] = a0 * sn + a1 * c;
       }
+      if (im.is_q && tempered) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          y0[i] *= q_mul;
+          y1[i] *= q_mul;
+        }
+      }
       *reinterpret_cast<uint4*>(at(im.j)) = pack8(y0);
       *reinterpret_cast<uint4*>(at(im.j + half)) = pack8(y1);
     } else {
-      if (im.bias) {
+      if (im.bias || (im.is_q && tempered)) {
+        const float mul = im.is_q ? q_mul : 1.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x0[i] += b0[i];
+        for (int i = 0; i < 8; ++i) x0[i] = (x0[i] + b0[i]) * mul;
         *reinterpret_cast<uint4*>(at(im.j)) = pack8(x0);
       } else {
         *reinterpret_cast<uint4*>(at(im.j)) = raw[0];
@@ -337,7 +358,7 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
                                  const void* seq_slot, const void* page_table, int max_blocks,
                                  int num_pages, const void* inv_freq, int rotary_dim, int rows,
                                  int H, int KVH, int hd, int hd_in, int vd_in, int interleaved,
-                                 float mscale, int dtype, void* stream) {
+                                 float mscale, float q_coef, int q_every, int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH >= 0 && hd > 0, "he_qkv_rope_cache: bad sizes");
   if (hd_in <= 0) hd_in = hd;
   if (vd_in <= 0) vd_in = hd;
@@ -362,7 +383,7 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
       in_stride, q_bias, k_bias, v_bias, bias_dtype,                                            \
       (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot,             \
       (const int32_t*)page_table, max_blocks, num_pages, (const float*)inv_freq, rotary_dim, H, \
-      KVH, hd, hd_in, vd_in, interleaved, mscale)
+      KVH, hd, hd_in, vd_in, interleaved, mscale, q_coef, q_every)
   const bool vec_ok = dtype == HE_BF16 &&
                       (q_bias == nullptr || bias_dtype == HE_BF16) &&
                       ((interleaved ? rotary_dim : rotary_dim >> 1) & 7) == 0 && ((hd - rotary_dim) & 7) == 0 &&
@@ -381,7 +402,8 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
         (const uint16_t*)k_in, (const uint16_t*)v_in, in_stride, (const uint16_t*)q_bias,
         (const uint16_t*)k_bias, (const uint16_t*)v_bias, (const int32_t*)positions,
         (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,
-        num_pages, (const float*)inv_freq, rotary_dim, rows, H, KVH, hd, hd_in, vd_in, interleaved, mscale, v_span);
+        num_pages, (const float*)inv_freq, rotary_dim, rows, H, KVH, hd, hd_in, vd_in, interleaved, mscale, v_span, q_coef,
+        q_every);
   } else if (dtype == HE_BF16) {
     ROPE_LAUNCH(bf16_t, bf16_t);
   } else {

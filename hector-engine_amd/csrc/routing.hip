@@ -1,0 +1,220 @@
+// A token's choice among experts, the experts' gated activation weighted by that choice, and the
+// combination of the two score maps of a differential attention head.
+#include "common.h"
+#include "hector_kernels.h"
+
+#define ROUTE_MAX_EXPERTS 1024
+
+// (value, index) maximum over the wavefront; among equal values the lowest index wins
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+  for (int m = 32; m >= 1; m >>= 1) {
+    const float ov = __shfl_xor(v, m);
+    const int oi = __shfl_xor(i, m);
+    if (ov > v || (ov == v && oi < i)) {
+      v = ov;
+      i = oi;
+    }
+  }
+}
+
+// One wavefront a row. logits [rows][E] fp32. s = softmax(logits) over all E outputs; the choice is made
+// on c = s + correction: the E outputs form `groups` equal groups of neighbours, a group counts by its
+// largest c, only the outputs of the `keep` best groups can be chosen (the others count as -inf), and
+// the `top` largest c among those are chosen. The weight of a chosen output is s * scale (not c, and
+// not renormalised). The last E - real outputs are experts without weights whose result is the input
+// itself: their weights are added up in column `real` of dense. dense [rows][real + 1] holds the
+// weight of every expert (0 where not chosen); ids / weights [rows][top] list the chosen ones.
+__global__ __launch_bounds__(64) void route_kernel(float* __restrict__ dense, int32_t* __restrict__ ids,
+                                                   float* __restrict__ weights, const float* __restrict__ logits,
+                                                   const void* __restrict__ correction, int c_dtype, int E, int real,
+                                                   int groups, int keep, int top, float scale) {
+  __shared__ float s_sh[ROUTE_MAX_EXPERTS];
+  __shared__ float c_sh[ROUTE_MAX_EXPERTS];
+  __shared__ float d_sh[ROUTE_MAX_EXPERTS + 1];
+  __shared__ float g_sh[ROUTE_MAX_EXPERTS];
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* z = logits + row * E;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += 64) {
+    const float v = expf(z[e] - mx);
+    s_sh[e] = v;
+    sum += v;
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.f / sum;
+  for (int e = lane; e < E; e += 64) {
+    const float s = s_sh[e] * inv;
+    s_sh[e] = s;
+    c_sh[e] = s + (correction ? load_param(correction, e, c_dtype) : 0.f);
+  }
+  for (int e = lane; e <= real; e += 64) d_sh[e] = 0.f;
+  __syncthreads();
+  const int size = E / groups;
+  if (keep < groups) {
+    for (int g = lane; g < groups; g += 64) {
+      float best = -INFINITY;
+      for (int i = 0; i < size; ++i) best = fmaxf(best, c_sh[g * size + i]);
+      g_sh[g] = best;
+    }
+    __syncthreads();
+    // the `keep` best groups are marked by +inf in g_sh, then the others' outputs are masked
+    for (int k = 0; k < keep; ++k) {
+      float v = -INFINITY;
+      int idx = 0x7fffffff;
+      for (int g = lane; g < groups; g += 64) {
+        const float gv = g_sh[g];
+        if (gv != INFINITY && (gv > v || (gv == v && g < idx))) {
+          v = gv;
+          idx = g;
+        }
+      }
+      wave_argmax(v, idx);
+      __syncthreads();
+      if (lane == 0 && idx < groups) g_sh[idx] = INFINITY;
+      __syncthreads();
+    }
+    for (int e = lane; e < E; e += 64)
+      if (g_sh[e / size] != INFINITY) c_sh[e] = -INFINITY;
+    __syncthreads();
+  }
+  for (int k = 0; k < top; ++k) {
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float cv = c_sh[e];
+      // a chosen output is marked by NaN, which no comparison takes
+      if (cv > v || (cv == v && e < idx)) {
+        v = cv;
+        idx = e;
+      }
+    }
+    wave_argmax(v, idx);
+    __syncthreads();
+    if (lane == 0) {
+      const bool found = idx < E;
+      const int e = found ? idx : 0;
+      const float w = found ? s_sh[e] * scale : 0.f;
+      if (found) {
+        c_sh[e] = NAN;
+        d_sh[e < real ? e : real] += w;
+      }
+      ids[row * top + k] = found ? e : -1;
+      weights[row * top + k] = w;
+    }
+    __syncthreads();
+  }
+  for (int e = lane; e <= real; e += 64) dense[row * (real + 1) + e] = d_sh[e];
+}
+
+extern "C" int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32, const void* logits_f32,
+                               const void* correction, int c_dtype, int rows, int E, int real, int groups, int keep,
+                               int top, float scale, void* stream) {
+  HE_REQUIRE(rows >= 0 && E > 0 && E <= ROUTE_MAX_EXPERTS && real >= 0 && real <= E,
+             "he_route_tokens: bad sizes E=%d real=%d (at most %d outputs)", E, real, ROUTE_MAX_EXPERTS);
+  HE_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups,
+             "he_route_tokens: %d outputs do not form %d equal groups of which %d are kept", E, groups, keep);
+  HE_REQUIRE(top > 0 && top <= keep * (E / groups), "he_route_tokens: %d chosen of %d kept outputs", top,
+             keep * (E / groups));
+  if (rows == 0) return 0;
+  route_kernel<<<rows, 64, 0, (hipStream_t)stream>>>((float*)dense_f32, (int32_t*)ids_i32, (float*)weights_f32,
+                                                     (const float*)logits_f32, correction, c_dtype, E, real, groups,
+                                                     keep, top, scale);
+  return he_check_launch("he_route_tokens");
+}
+
+// out [rows][real * I + extra]: column e * I + i = act(gate, up) * dense[row][e] with gate and up the
+// columns 2 (e I + i) and 2 (e I + i) + 1 of gate_up (a fused weight whose rows alternate gate and up),
+// act as he_gated_act; the last `extra` columns = dense[row][real] * h[row][:] (the share of the
+// experts whose result is their input). A product over these columns with the experts' down
+// matrices side by side (and an identity block for the extra columns) is the weighted sum of the
+// chosen experts' results.
+template <typename T, bool CLAMPED>
+__global__ void routed_act_kernel(T* __restrict__ out, const T* __restrict__ gate_up, const float* __restrict__ dense,
+                                  const T* __restrict__ h, int real, int I, int extra, GatedAct act) {
+  const int64_t row = blockIdx.y;
+  const int cols = real * I + extra;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= cols) return;
+  const float* d = dense + row * (real + 1);
+  float v;
+  if (j < real * I) {
+    const float w = d[j / I];
+    const T* gu = gate_up + row * (int64_t)(2 * real * I) + 2 * j;
+    // an expert that was not chosen gives exact zeros, whatever its rows hold
+    v = w == 0.f ? 0.f : he_gated_act<CLAMPED>(to_float(gu[0]), to_float(gu[1]), act) * w;
+  } else {
+    const float w = d[real];
+    v = w == 0.f ? 0.f : w * to_float(h[row * (int64_t)extra + (j - real * I)]);
+  }
+  out[row * (int64_t)cols + j] = from_float<T>(v);
+}
+
+extern "C" int he_routed_act(void* out, const void* gate_up, const void* dense_f32, const void* h, int rows, int real,
+                             int I, int extra, int dtype, float alpha, float limit, float up_shift, void* stream) {
+  HE_REQUIRE(rows >= 0 && real >= 0 && I > 0 && extra >= 0 && (int64_t)real * I + extra > 0, "he_routed_act: bad sizes");
+  HE_REQUIRE(extra == 0 || h != nullptr, "he_routed_act: the input rows are missing");
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_routed_act: unknown dtype %d", dtype);
+  if (rows == 0) return 0;
+  const int cols = real * I + extra;
+  const dim3 grid((cols + 255) / 256, rows);
+  hipStream_t s = (hipStream_t)stream;
+  const bool clamped = limit > 0.f || alpha != 1.f || up_shift != 0.f;
+  const GatedAct act = {alpha, limit > 0.f ? limit : INFINITY, up_shift};
+#define ACT_LAUNCH(T, CL)                                                                                      \
+  routed_act_kernel<T, CL><<<grid, 256, 0, s>>>((T*)out, (const T*)gate_up, (const float*)dense_f32, (const T*)h, real, \
+                                                I, extra, act)
+  if (dtype == HE_BF16) {
+    if (clamped) ACT_LAUNCH(bf16_t, true); else ACT_LAUNCH(bf16_t, false);
+  } else {
+    if (clamped) ACT_LAUNCH(float, true); else ACT_LAUNCH(float, false);
+  }
+#undef ACT_LAUNCH
+  return he_check_launch("he_routed_act");
+}
+
+// Differential attention's last step. attn [rows][2 H][hd] holds, for kv head g and its R = H / G
+// query heads, first the R outputs of score map 1 and then the R outputs of map 2 (head order
+// [g][map][r]); out [rows][H][vd], head h = g R + r:
+//   o = a1 - lambda a2;  out = o / sqrt(mean(o^2) + eps) * post
+// over the vd values of a head (no learned gain). One wavefront a (row, head).
+template <typename T>
+__global__ __launch_bounds__(64) void diff_heads_kernel(T* __restrict__ out, const T* __restrict__ attn, int H, int G,
+                                                        int hd, int vd, float lambda, float post, float eps) {
+  const int64_t row = blockIdx.y;
+  const int h = blockIdx.x;
+  const int R = H / G;
+  const int g = h / R, r = h - g * R;
+  const T* a1 = attn + (row * 2 * H + (int64_t)(2 * g) * R + r) * hd;
+  const T* a2 = a1 + (int64_t)R * hd;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < vd; i += 64) {
+    const float o = fmaf(-lambda, to_float(a2[i]), to_float(a1[i]));
+    sq = fmaf(o, o, sq);
+  }
+  sq = wave_sum(sq);
+  const float mul = post / sqrtf(sq / (float)vd + eps);
+  T* dst = out + (row * H + h) * vd;
+  for (int i = threadIdx.x; i < vd; i += 64) {
+    const float o = fmaf(-lambda, to_float(a2[i]), to_float(a1[i]));
+    dst[i] = from_float<T>(o * mul);
+  }
+}
+
+extern "C" int he_diff_heads(void* out, const void* attn, int rows, int H, int G, int hd, int vd, float lambda,
+                             float post, float eps, int dtype, void* stream) {
+  HE_REQUIRE(rows >= 0 && H > 0 && G > 0 && H % G == 0 && vd > 0 && vd <= hd, "he_diff_heads: bad sizes H=%d G=%d hd=%d vd=%d",
+             H, G, hd, vd);
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_diff_heads: unknown dtype %d", dtype);
+  if (rows == 0) return 0;
+  const dim3 grid(H, rows);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HE_BF16)
+    diff_heads_kernel<bf16_t><<<grid, 64, 0, s>>>((bf16_t*)out, (const bf16_t*)attn, H, G, hd, vd, lambda, post, eps);
+  else
+    diff_heads_kernel<float><<<grid, 64, 0, s>>>((float*)out, (const float*)attn, H, G, hd, vd, lambda, post, eps);
+  return he_check_launch("he_diff_heads");
+}

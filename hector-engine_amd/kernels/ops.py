@@ -487,7 +487,7 @@ def splitk_reduce(out, partial, bias, M: int, splits: int) -> None:
 def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, positions, row_seq,
                    seq_slot, page_table, inv_freq, rotary_dim: int, rows: int, H: int, KVH: int,
                    hd: int, write_kv: bool, *, key_dim: int = 0, value_dim: int = 0,
-                   interleaved: bool = False, mscale: float = 1.0) -> None:
+                   interleaved: bool = False, mscale: float = 1.0, q_temp=None) -> None:
     """qkv: [rows, q_cols + kv_cols + v_cols (+ more)] projected rows without bias; bias (optional)
     covers those columns. Rotated q goes to q_out [rows, H*hd]; k, v go into the pools at
     (slot, position) when write_kv. hd is the head size of q_out and of the cache pages; key_dim and
@@ -546,7 +546,144 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
         base, k_in, v_in, width, qb, kb, vb, bias_code, positions.data_ptr(), row_seq.data_ptr(),
         seq_slot.data_ptr(), _ptr(page_table) if write_kv else None, max_blocks, num_pages,
         _ptr(inv_freq) if rotary_dim else None, rotary_dim, rows, H, KVH if write_kv else 0, hd,
-        kd, vd, int(interleaved), float(mscale), dtype_code(q_out.dtype), _stream()))
+        kd, vd, int(interleaved), float(mscale), float(q_temp[0]) if q_temp else 0.0,
+        int(q_temp[1]) if q_temp else 0, dtype_code(q_out.dtype), _stream()))
+
+
+@_op("conv_state")
+def conv_state(out, x, taps, bias, state, positions, row_seq, seq_slot, seq_start, cu_seqlens,
+               rows: int, num_seqs: int, all_single: bool) -> None:
+    """out[rows, C] = silu(causal convolution per channel of x + bias), the taps' last column on the
+    row's own input; the inputs before a step's first row come from the sequence's row of `state`
+    (uint8 [slots, bytes], fp32 [K-1][C] at its start), which is then moved on. x: a view [rows, C]
+    of wider rows (unit stride along C)."""
+    C, K = taps.shape
+    _need(out, "out", x.dtype, (None, C))
+    _need(taps, "taps")
+    _need(bias, "bias", taps.dtype, (C,))
+    if x.dim() != 2 or x.shape[1] != C or x.stride(1) != 1 or x.shape[0] < rows or out.shape[0] < rows:
+        raise ValueError("conv_state: x must be [rows, C] with unit stride along C")
+    if state.dtype != torch.uint8 or state.dim() != 2 or state.stride(1) != 1:
+        raise ValueError("conv_state: state must be uint8 [slots, bytes]")
+    for name, t, n in (("positions", positions, rows), ("row_seq", row_seq, rows), ("seq_slot", seq_slot, num_seqs),
+                       ("seq_start", seq_start, num_seqs), ("cu_seqlens", cu_seqlens, num_seqs + 1)):
+        _need(t, name, torch.int32)
+        if t.numel() < n:
+            raise ValueError(f"conv_state: {name} shorter than the step")
+    if state.shape[1] < 4 * (K - 1) * C:
+        raise ValueError("conv_state: the state rows are too short")
+    L = _lib.load()
+    _lib.check(L.he_conv_state(out.data_ptr(), x.data_ptr(), x.stride(0), taps.data_ptr(), bias.data_ptr(),
+                               dtype_code(taps.dtype), state.data_ptr(), state.stride(0), positions.data_ptr(),
+                               row_seq.data_ptr(), seq_slot.data_ptr(), seq_start.data_ptr(), cu_seqlens.data_ptr(),
+                               rows, num_seqs, C, K, int(all_single), dtype_code(x.dtype), _stream()))
+
+
+def ssm_state_floats(R: int, P: int, N: int) -> int:
+    """Floats of a sequence's scan state (the state dims padded to the threads' share)."""
+    return int(_lib.load().he_ssm_state_floats(R, P, N))
+
+
+@_op("ssm_scan")
+def ssm_scan(y, xbc, dt, dt_bias, a_log, d_skip, state, state_offset: int, cu_seqlens, seq_slot,
+             rows: int, num_seqs: int, R: int, Q: int, N: int, P: int) -> None:
+    """y (fp32 [rows, R P]) = the selective scan of xbc [rows, R P + 2 Q N] (x, then B, then C) with step
+    sizes softplus(dt + dt_bias) (dt: a view [rows, R] of wider rows), per head r the decay
+    exp(-exp(a_log_r) dt) and the skip d_skip_r; the state [R][P][N'] lives at byte state_offset of a
+    sequence's row of `state` and is carried on."""
+    C = R * P + 2 * Q * N
+    _need(y, "y", torch.float32, (None, R * P))
+    _need(xbc, "xbc", None, (None, C))
+    if dt.dtype != xbc.dtype or dt.dim() != 2 or dt.shape[1] != R or dt.stride(1) != 1:
+        raise ValueError("ssm_scan: dt must be a [rows, R] view in xbc's dtype")
+    for name, t in (("dt_bias", dt_bias), ("a_log", a_log), ("d_skip", d_skip)):
+        _need(t, name, dt_bias.dtype, (R,))
+    if y.shape[0] < rows or xbc.shape[0] < rows or dt.shape[0] < rows:
+        raise ValueError("ssm_scan: buffers smaller than the row count")
+    if state.dtype != torch.uint8 or state.dim() != 2 or state.stride(1) != 1 \
+            or state.shape[1] < state_offset + 4 * ssm_state_floats(R, P, N):
+        raise ValueError("ssm_scan: state must be uint8 [slots, bytes] with room for the scan's state")
+    _need(cu_seqlens, "cu_seqlens", torch.int32)
+    _need(seq_slot, "seq_slot", torch.int32)
+    if cu_seqlens.numel() < num_seqs + 1 or seq_slot.numel() < num_seqs:
+        raise ValueError("ssm_scan: metadata shorter than the step")
+    L = _lib.load()
+    _lib.check(L.he_ssm_scan(y.data_ptr(), xbc.data_ptr(), dt.data_ptr(), dt.stride(0), dt_bias.data_ptr(),
+                             a_log.data_ptr(), d_skip.data_ptr(), dtype_code(dt_bias.dtype), state.data_ptr(),
+                             state.stride(0), state_offset, cu_seqlens.data_ptr(), seq_slot.data_ptr(), rows,
+                             num_seqs, R, Q, N, P, dtype_code(xbc.dtype), _stream()))
+
+
+@_op("gated_group_norm")
+def gated_group_norm(out, y, z, weight, rows: int, parts: int, eps: float) -> None:
+    """out[rows, W] = (y * silu(z)), each of `parts` equal stretches of a row divided by its own root mean
+    square, times weight. y fp32 [rows, W]; z a view [rows, W] of wider rows in out's dtype."""
+    W = weight.shape[0]
+    _need(out, "out", None, (None, W))
+    _need(y, "y", torch.float32, (None, W))
+    _need(weight, "weight")
+    if z.dtype != out.dtype or z.dim() != 2 or z.shape[1] != W or z.stride(1) != 1:
+        raise ValueError("gated_group_norm: z must be a [rows, W] view in out's dtype")
+    if min(out.shape[0], y.shape[0], z.shape[0]) < rows or W % parts:
+        raise ValueError("gated_group_norm: buffers smaller than the row count, or parts that do not divide the width")
+    L = _lib.load()
+    _lib.check(L.he_gated_group_norm(out.data_ptr(), y.data_ptr(), z.data_ptr(), z.stride(0), weight.data_ptr(),
+                                     dtype_code(weight.dtype), rows, W, parts, float(eps), dtype_code(out.dtype),
+                                     _stream()))
+
+
+@_op("route_tokens")
+def route_tokens(dense, ids, weights, logits, correction, rows: int, real: int, groups: int, keep: int,
+                 top: int, scale: float) -> None:
+    """The choice of `top` of E router outputs per row (logits fp32 [rows, E]): softmax scores s, the choice on
+    s + correction inside the `keep` best of `groups` equal groups, weights s * scale. dense (fp32
+    [rows, real + 1]): each expert's weight or 0, the outputs from `real` on added up in the last column;
+    ids (int32) and weights (fp32) [rows, top]: the chosen outputs."""
+    E = logits.shape[-1]
+    _need(logits, "logits", torch.float32, (None, E))
+    _need(dense, "dense", torch.float32, (None, real + 1))
+    _need(ids, "ids", torch.int32, (None, top))
+    _need(weights, "weights", torch.float32, (None, top))
+    if correction is not None:
+        _need(correction, "correction", None, (E,))
+    if min(logits.shape[0], dense.shape[0], ids.shape[0], weights.shape[0]) < rows:
+        raise ValueError("route_tokens: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_route_tokens(dense.data_ptr(), ids.data_ptr(), weights.data_ptr(), logits.data_ptr(),
+                                 _ptr(correction), dtype_code(correction.dtype) if correction is not None else F32,
+                                 rows, E, real, groups, keep, top, float(scale), _stream()))
+
+
+@_op("routed_act")
+def routed_act(out, gate_up, dense, h, rows: int, real: int, inter: int, *, alpha: float = 1.0,
+               limit: float = 0.0, up_shift: float = 0.0) -> None:
+    """out[rows, real * inter + extra]: the experts' gated activations (gate_up [rows, 2 real inter], gate and
+    up alternating) times their weights dense[row, e]; the last extra = h.shape[1] columns (h None: none)
+    are dense[row, real] * h."""
+    extra = 0 if h is None else h.shape[1]
+    _need(out, "out", None, (None, real * inter + extra))
+    _need(gate_up, "gate_up", out.dtype, (None, 2 * real * inter))
+    _need(dense, "dense", torch.float32, (None, real + 1))
+    if h is not None:
+        _need(h, "h", out.dtype)
+    if min(out.shape[0], gate_up.shape[0], dense.shape[0], rows if h is None else h.shape[0]) < rows:
+        raise ValueError("routed_act: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_routed_act(out.data_ptr(), gate_up.data_ptr(), dense.data_ptr(), _ptr(h), rows, real, inter,
+                               extra, dtype_code(out.dtype), float(alpha), float(limit), float(up_shift), _stream()))
+
+
+@_op("diff_heads")
+def diff_heads(out, attn, rows: int, H: int, G: int, hd: int, vd: int, lam: float, post: float, eps: float) -> None:
+    """out[rows, H, vd] = rms(a1 - lam * a2) * post per head, a1 and a2 the outputs of the two score maps in
+    attn [rows, 2 H, hd] (head order [kv head][map][query head of the group])."""
+    _need(attn, "attn")
+    _need(out, "out", attn.dtype)
+    if attn.numel() < rows * 2 * H * hd or out.numel() < rows * H * vd:
+        raise ValueError("diff_heads: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_diff_heads(out.data_ptr(), attn.data_ptr(), rows, H, G, hd, vd, float(lam), float(post),
+                               float(eps), dtype_code(out.dtype), _stream()))
 
 
 def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):

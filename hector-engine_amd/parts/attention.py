@@ -21,7 +21,17 @@ Options of the same part, each off unless its parameter says otherwise:
               key and no value, is not scaled and counts once.
   head_gate   head h's output is multiplied by sigmoid(g_h), g = Wg n with one row of Wg a head;
               the rows of Wg ride behind q||k||v in the one product.
-  names       the suffixes of its tensors (q, k, v, o, q_bias, k_bias, v_bias, o_bias, sinks, gate).
+  q_temp      {coef, every}: the q of position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).
+  score_maps  2: differential attention. A head has two queries and a kv head two keys (the rows of
+              the q and k matrices lie head by head as [map 1, map 2]); each map is a softmax attention
+              of its own over the same values, a1 and a2, and the head's output is
+              rms(a1 - lambda * a2) * (1 - diff) over its value_dim values (no gain, eps `diff_eps`), with
+              lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff from four stored vectors of head_dim and the
+              constant `diff`. The kernels see 2 H heads over 2 KVH kv heads: the rows of q are reordered
+              so that the heads of one (kv head, map) are neighbours, and the value rows of a kv head
+              stand once for each of its maps; ops.diff_heads then joins the pairs.
+  names       the suffixes of its tensors (q, k, v, o, q_bias, k_bias, v_bias, o_bias, sinks, gate,
+              lq1, lk1, lq2, lk2).
 """
 from __future__ import annotations
 
@@ -36,7 +46,8 @@ from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, Ste
 
 _NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
           "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
-          "sinks": "sinks", "gate": "gate.weight"}
+          "sinks": "sinks", "gate": "gate.weight", "lq1": "lambda_q1", "lk1": "lambda_k1", "lq2": "lambda_q2",
+          "lk2": "lambda_k2"}
 from .linear import Linear
 
 
@@ -78,6 +89,18 @@ class Attention(Mixer):
         self.chunk = param(params, "chunk", int, 0)
         self.has_sinks = param(params, "sinks", bool, False)
         self.head_gate = param(params, "head_gate", bool, False)
+        self.maps = param(params, "score_maps", int, 1)
+        self.diff = param(params, "diff", float, 0.0)
+        self.diff_eps = param(params, "diff_eps", float, 1e-6)
+        self.lam = 0.0                      # lambda of a differential attention, from its four vectors (bind)
+        qt = param(params, "q_temp", dict, None)
+        self.q_temp = None if not qt else (float(qt["coef"]), int(qt["every"]))
+        if self.maps not in (1, 2) or (self.maps == 2 and self.head_gate):
+            raise ValueError(f"attention: score_maps {self.maps} must be 1 or 2 (and 2 goes without head gates)")
+        if self.q_temp is not None and self.q_temp[1] <= 0:
+            raise ValueError(f"attention: q_temp.every {self.q_temp[1]} must be positive")
+        # the heads as the kernels count them: a differential head is two, one a score map
+        self.Hk, self.KVHk = self.H * self.maps, self.KVH * self.maps
         names = param(params, "names", dict, {})
         self._names = {k: tensor_name(prefix, names, k, d) for k, d in _NAMES.items()}
         if self.H % self.KVH:
@@ -99,28 +122,31 @@ class Attention(Mixer):
         self._chosen_version = -1
         self.fast = mfma and self.pd % 16 == 0 and self.pd <= 256 and self.scale > 0   # else the plain kernel
         # what the fused one-token kernel and the kernels without these options do not take
-        self.extras = self.chunk > 0 or self.has_sinks or self.head_gate
+        self.extras = self.chunk > 0 or self.has_sinks or self.head_gate or self.maps > 1 or self.q_temp is not None
 
     def children(self):
         return [self.position]
 
     def kv_need(self):
         # pages in the order the attention kernels read their operands
-        return KVNeed(self.KVH, self.pd, self.window, k_page_elems=kv_layout.k_page_elems(self.pd),
+        return KVNeed(self.KVHk, self.pd, self.window, k_page_elems=kv_layout.k_page_elems(self.pd),
                       v_page_elems=kv_layout.v_page_elems(self.pd), chunk=self.chunk)
 
     def tensor_specs(self):
         n, hd, vd = self._names, self.hd, self.vd
-        specs = {n["q"]: TensorSpec((self.H * hd, self.hidden)),
+        specs = {n["q"]: TensorSpec((self.Hk * hd, self.hidden)),
                  n["o"]: TensorSpec((self.hidden, self.H * vd))}
         if self.kv_projection:
-            specs[n["k"]] = TensorSpec((self.KVH * hd, self.hidden))
+            specs[n["k"]] = TensorSpec((self.KVHk * hd, self.hidden))
             specs[n["v"]] = TensorSpec((self.KVH * vd, self.hidden))
         if self.qkv_bias:
-            specs[n["q_bias"]] = TensorSpec((self.H * hd,))
+            specs[n["q_bias"]] = TensorSpec((self.Hk * hd,))
             if self.kv_projection:
-                specs[n["k_bias"]] = TensorSpec((self.KVH * hd,))
+                specs[n["k_bias"]] = TensorSpec((self.KVHk * hd,))
                 specs[n["v_bias"]] = TensorSpec((self.KVH * vd,))
+        if self.maps == 2:
+            for key in ("lq1", "lk1", "lq2", "lk2"):
+                specs[n[key]] = TensorSpec((hd,), ("normal", 0.1))
         if self.out_bias:
             specs[n["o_bias"]] = TensorSpec((self.hidden,))
         if self.has_sinks:
@@ -133,7 +159,7 @@ class Attention(Mixer):
     def bind(self, tensors):
         p, n = self.prefix, self._names
         names = ["q"] + (["k", "v"] if self.kv_projection else [])
-        ws = [tensors.pop(n[x]) for x in names]
+        ws = [self._by_map(x, tensors.pop(n[x])) for x in names]
         gate_w = tensors.pop(n["gate"]) if self.head_gate else None
         if gate_w is not None:
             ws.append(gate_w)          # the gate's rows ride behind q||k||v: one product
@@ -145,7 +171,7 @@ class Attention(Mixer):
         w = torch.cat(ws, 0).contiguous() if len(ws) > 1 else ws[0]
         b = None
         if self.qkv_bias:
-            bs = [tensors.pop(n[x + "_bias"]) for x in names]
+            bs = [self._by_map(x, tensors.pop(n[x + "_bias"])) for x in names]
             if len({x.dtype for x in bs}) != 1:
                 raise TypeError(f"{p}q/k/v biases are stored in different dtypes")
             b = torch.cat(bs, 0).contiguous() if len(bs) > 1 else bs[0]
@@ -156,7 +182,7 @@ class Attention(Mixer):
             return torch.cat([bias, torch.zeros(rows - bias.numel(), dtype=bias.dtype, device=bias.device)])
 
         self.qkv = Linear(w, bias_for(b, w.shape[0]))
-        q_rows = self.H * self.hd
+        q_rows = self.Hk * self.hd
         if gate_w is not None and self.kv_projection:
             spare = -(q_rows + self.H) % 8
             self.q_only = Linear(torch.cat([ws[0], gate_w, torch.zeros((spare, gate_w.shape[1]), dtype=gate_w.dtype,
@@ -167,7 +193,10 @@ class Attention(Mixer):
                                  None if b is None else bias_for(b[:q_rows], w.shape[0] if gate_w is not None else q_rows))
         del ws
         wo = tensors[n["o"]]
-        if self.pd != self.vd:
+        if self.maps == 2:
+            f = lambda key: tensors[n[key]].to(device="cpu", dtype=torch.float32)
+            self.lam = float(torch.exp((f("lq1") * f("lk1")).sum()) - torch.exp((f("lq2") * f("lk2")).sum())) + self.diff
+        if self.pd != self.vd and self.maps == 1:
             # zero columns where the attention's output holds the padding of a head
             padded = torch.zeros((self.hidden, self.H, self.pd), dtype=wo.dtype, device=wo.device)
             padded[:, :, :self.vd] = wo.view(self.hidden, self.H, self.vd)
@@ -176,6 +205,29 @@ class Attention(Mixer):
         if self.has_sinks:
             self.sinks = tensors[n["sinks"]]
         self.position.bind(tensors)
+
+    def _by_map(self, which: str, t: torch.Tensor) -> torch.Tensor:
+        """A differential attention's stored rows (or bias) as the kernels' heads read them: q from
+        [head][map] to [kv head][map][head of the group]; k is stored [kv head][map] already; the
+        value rows of a kv head once for each of its two maps."""
+        if self.maps == 1 or which == "k":
+            return t
+        rest = t.shape[1:]
+        if which == "q":
+            G, R = self.KVH, self.H // self.KVH
+            return t.reshape(G, R, 2, self.hd, *rest).transpose(1, 2).reshape(t.shape).contiguous()
+        return t.reshape(self.KVH, 1, self.vd, *rest).expand(self.KVH, 2, self.vd, *rest).reshape(
+            2 * t.shape[0], *rest).contiguous()
+
+    def _project(self, out, rows: int, ctx: StepContext):
+        """The output product behind the attention kernels (a differential attention joins its pairs
+        of heads first)."""
+        if self.maps == 2:
+            mixed = ctx.alloc((rows, self.H * self.vd))
+            ops.diff_heads(mixed, out, rows, self.H, self.KVH, self.pd, self.vd, self.lam, 1.0 - self.diff,
+                           self.diff_eps)
+            out = mixed
+        return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
 
     def forward(self, x, ctx: StepContext, cache: LayerCache):
         if cache.writes and not self.kv_projection:
@@ -225,7 +277,7 @@ class Attention(Mixer):
     def _encoded_q(self, x, ctx: StepContext, cache: LayerCache):
         """(q with bias and position encoding, after the new keys and values went into the cache;
         the heads' gates as a view of the projection's rows, or None)."""
-        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
+        rows, H, KVH, hd = ctx.rows, self.Hk, self.KVHk, self.hd
         writes = cache.writes
         proj = self.qkv if writes else self.q_only
         rot = self.position.rotary()
@@ -244,7 +296,7 @@ class Attention(Mixer):
                            proj.bias if fused_bias else None, ctx.positions, ctx.row_seq,
                            ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, self.pd, writes,
                            key_dim=hd, value_dim=self.vd, interleaved=self.position.interleaved,
-                           mscale=self.position.mscale)
+                           mscale=self.position.mscale, q_temp=self.q_temp)
         gate = None
         if self.head_gate:
             at = H * hd + (KVH * (hd + self.vd) if writes else 0)
@@ -253,7 +305,7 @@ class Attention(Mixer):
 
     def _run_plain(self, x, ctx: StepContext, cache: LayerCache):
         """The plain kernel: one fixed order per (query, head), in the precision of the cache."""
-        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.pd
+        rows, H, KVH, hd = ctx.rows, self.Hk, self.KVHk, self.pd
         q, gate = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
         floats = ops.attention_plain_workspace_floats(rows, H, hd, ctx.most_keys, self.window, self.chunk)
@@ -261,11 +313,11 @@ class Attention(Mixer):
         ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                             ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
                             self.scale, ctx.most_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate)
-        return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
+        return self._project(out, rows, ctx)
 
     def _run_mfma_one_token(self, x, ctx: StepContext, cache: LayerCache):
         """One-token steps of the head sizes and encodings the fused kernel does not take."""
-        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.pd
+        rows, H, KVH, hd = ctx.rows, self.Hk, self.KVHk, self.pd
         q, gate = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
         floats = ops.attention_decode_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
@@ -273,11 +325,11 @@ class Attention(Mixer):
         ops.attention_decode(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                              ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
                              self.scale, ctx.max_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate)
-        return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
+        return self._project(out, rows, ctx)
 
     def _run_mfma_prompt(self, x, ctx: StepContext, cache: LayerCache):
         """Prompt steps and mixed steps."""
-        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.pd
+        rows, H, KVH, hd = ctx.rows, self.Hk, self.KVHk, self.pd
         q, gate = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
         # few queries against many keys (a continuation of a long sequence): the keys in parts
@@ -297,7 +349,7 @@ class Attention(Mixer):
                               ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
                               rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws,
                               chunk=self.chunk, sinks=self.sinks, gate=gate)
-        return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
+        return self._project(out, rows, ctx)
 
 
 _BF16 = (torch.bfloat16,)

@@ -16,13 +16,15 @@ class RMSNorm(Norm):
         super().__init__(prefix, env)
         self.size = param(params, "size", int)
         self.eps = param(params, "eps", float)
+        # names: the suffix of its tensor (weight)
+        self._name = tensor_name(prefix, param(params, "names", dict, {}), "weight", "weight")
         self.weight: torch.Tensor | None = None
 
     def tensor_specs(self):
-        return {self.prefix + "weight": TensorSpec((self.size,), ("gain", 1.0, 0.1))}
+        return {self._name: TensorSpec((self.size,), ("gain", 1.0, 0.1))}
 
     def bind(self, tensors):
-        self.weight = tensors[self.prefix + "weight"]
+        self.weight = tensors[self._name]
 
     def carried(self):
         return self.weight, self.eps
