@@ -218,3 +218,14 @@ def forward(cfg, w, tokens, carry=None, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return (rms(x, eps) * w["final.norm"]) @ w["embed"].T, carry
+
+
+def greedy(cfg, w, prompt, steps: int) -> list[int]:
+    """`steps` tokens after `prompt`, each the argmax of the last logits (lowest id on ties)."""
+    logits, carry = forward(cfg, w, list(prompt))
+    out = []
+    for _ in range(steps):
+        t = int(torch.argmax(logits[-1]))
+        out.append(t)
+        logits, carry = forward(cfg, w, [t], carry)
+    return out

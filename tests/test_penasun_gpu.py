@@ -1,0 +1,606 @@
+"""Penasun on the GPU against the plain implementation (tests/plain/penasun_plain.py): each new
+mechanism alone at its kernel, fed in portions and in batches, with inputs planted so that a lost
+state, a choice outside the kept groups or a wrong head pairing shows; then whole models of
+several shapes and layer orders through the engine's step function, cut and batched in many ways,
+in 32-bit and in bfloat16; and greedy generation through the library's own entry point."""
+import json
+import math
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests.helpers import argmax_agrees_where_clear, close, rand_ids
+from tests.plain import penasun_plain as P
+from tests.test_kernels_gpu import dev, rnd
+from tests.test_penasun_cpu import attn, layer, moe, scan
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import hector_engine_amd  # noqa: F401
+    from hector_engine_amd.kernels import ops as o
+    return o
+
+
+def i32(values):
+    return torch.tensor(values, dtype=torch.int32, device="cuda")
+
+
+def step_meta(q_lens, starts, slots):
+    """positions, row_seq, seq_slot, seq_start, cu_seqlens of a packed step."""
+    positions, row_seq, cu = [], [], [0]
+    for s, (n, at) in enumerate(zip(q_lens, starts)):
+        positions += list(range(at, at + n))
+        row_seq += [s] * n
+        cu.append(cu[-1] + n)
+    return i32(positions), i32(row_seq), i32(slots), i32(starts), i32(cu)
+
+
+# a schedule of steps over three sequences: (sequence, new tokens) per step; lengths 71, 9 and 140
+SCHEDULE = [[(0, 3), (1, 1), (2, 64)], [(0, 1), (1, 1), (2, 1)], [(0, 2), (2, 2)], [(1, 7), (2, 70)],
+            [(0, 64)], [(0, 1), (2, 1)], [(2, 2)]]
+LENGTHS = [71, 9, 140]
+
+
+def run_schedule(slots, per_step):
+    """Feeds SCHEDULE; per_step(seqs, q_lens, starts, row ranges) runs one step."""
+    done = [0, 0, 0]
+    for step in SCHEDULE:
+        seqs = [s for s, _ in step]
+        q_lens = [n for _, n in step]
+        starts = [done[s] for s in seqs]
+        per_step(seqs, q_lens, starts, [slots[s] for s in seqs])
+        for s, n in step:
+            done[s] += n
+    assert done == LENGTHS
+
+
+# ------------------------------------------------------------------ convolution with carried inputs
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,K", [(10, 1), (37, 2), (300, 4), (64, 7)])
+def test_convolution_in_portions_and_batches_equals_the_whole(ops, dtype, C, K):
+    dt = TORCH[dtype]
+    u = [rnd(n, C + 5, seed=3 + i).to(dt) for i, n in enumerate(LENGTHS)]       # rows wider than the channels read
+    taps, bias = rnd(C, K, seed=1, scale=0.5).to(dt), rnd(C, seed=2).to(dt)
+    want = [P.causal_conv(x[:, 2:2 + C].double(), taps.double(), bias.double())[0] for x in u]
+    slots = [4, 0, 2]                                                          # not in order, with gaps
+    state = torch.zeros(6, 4 * (K - 1) * C + 64, dtype=torch.uint8, device="cuda")
+    state[:, 4 * (K - 1) * C:] = 77                                            # what lies behind is not touched
+    got = [torch.zeros(n, C, dtype=torch.float64) for n in LENGTHS]
+
+    def per_step(seqs, q_lens, starts, sl):
+        x = torch.cat([u[s][at:at + n] for s, n, at in zip(seqs, q_lens, starts)])
+        rows = x.shape[0]
+        out = torch.empty(rows, C, dtype=dt, device="cuda")
+        ops.conv_state(out, dev(x)[:, 2:2 + C], dev(taps), dev(bias), state, *step_meta(q_lens, starts, sl),
+                       rows, len(seqs), all(n == 1 for n in q_lens))
+        at = 0
+        for s, n, st in zip(seqs, q_lens, starts):
+            got[s][st:st + n] = out[at:at + n].cpu().double()
+            at += n
+
+    run_schedule(slots, per_step)
+    tol = 2e-6 if dtype == "float32" else 2 ** -7
+    for g, w in zip(got, want):
+        assert torch.allclose(g, w, rtol=tol, atol=tol)
+    assert bool((state[:, 4 * (K - 1) * C:] == 77).all())
+    assert bool((state[[1, 3, 5]][:, :4 * (K - 1) * C] == 0).all())            # rows of other slots stay as they were
+
+
+# ------------------------------------------------------------------ selective scan
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("R,Q,N,P_", [(3, 1, 20, 12), (4, 4, 96, 40), (2, 2, 16, 64), (8, 2, 128, 72), (1, 1, 5, 3)])
+def test_scan_in_portions_and_batches_equals_the_whole(ops, dtype, R, Q, N, P_):
+    tdt = TORCH[dtype]
+    inner, C = R * P_, R * P_ + 2 * Q * N
+    xbc = [rnd(n, C, seed=10 + i).to(tdt) for i, n in enumerate(LENGTHS)]
+    dts = [rnd(n, R + 3, seed=20 + i).to(tdt) for i, n in enumerate(LENGTHS)]
+    dt_bias, a_log, d_skip = rnd(R, seed=30, scale=0.5).to(tdt) - 1, rnd(R, seed=31, scale=0.5).to(tdt), rnd(R, seed=32).to(tdt)
+    want = []
+    for x, d in zip(xbc, dts):
+        T = x.shape[0]
+        step = P.softplus(d[:, 1:1 + R].double() + dt_bias.double())
+        y, _ = P.selective_scan(x[:, :inner].double().reshape(T, R, P_), x[:, inner:inner + Q * N].double().reshape(T, Q, N),
+                                x[:, inner + Q * N:].double().reshape(T, Q, N), step, a_log.double(), d_skip.double())
+        want.append(y.reshape(T, inner))
+    offset = 48
+    floats = ops.ssm_state_floats(R, P_, N)
+    state = torch.zeros(5, offset + 4 * floats + 16, dtype=torch.uint8, device="cuda")
+    slots = [3, 1, 0]
+    got = [torch.zeros(n, inner, dtype=torch.float64) for n in LENGTHS]
+
+    def per_step(seqs, q_lens, starts, sl):
+        x = torch.cat([xbc[s][at:at + n] for s, n, at in zip(seqs, q_lens, starts)])
+        d = torch.cat([dts[s][at:at + n] for s, n, at in zip(seqs, q_lens, starts)])
+        rows = x.shape[0]
+        y = torch.full((rows, inner), float("nan"), device="cuda")
+        _, _, seq_slot, _, cu = step_meta(q_lens, starts, sl)
+        ops.ssm_scan(y, dev(x), dev(d)[:, 1:1 + R], dev(dt_bias), dev(a_log), dev(d_skip), state, offset, cu, seq_slot,
+                     rows, len(seqs), R, Q, N, P_)
+        at = 0
+        for s, n, st in zip(seqs, q_lens, starts):
+            got[s][st:st + n] = y[at:at + n].cpu().double()
+            at += n
+
+    run_schedule(slots, per_step)
+    for g, w in zip(got, want):
+        assert torch.allclose(g, w, rtol=3e-5, atol=3e-5 * w.abs().max().item())
+    assert bool((state[:, :offset] == 0).all()) and bool((state[[2, 4]] == 0).all())
+
+
+def test_a_state_that_was_lost_shows(ops):
+    """One early token writes a large state that decays slowly; hundreds of tokens later the output is
+    still that state's, whether the tokens came at once or one by one."""
+    R, Q, N, P_ = 2, 1, 8, 16
+    inner, C, T = R * P_, R * P_ + 2 * N, 300
+    x = torch.zeros(T, C)
+    x[:, inner:] = 0.01 * rnd(T, 2 * N, seed=1)
+    x[5, :inner] = 50.0
+    x[5, inner:inner + N] = 1.0
+    x[:, inner + N:] += 1.0                                  # every token reads the state
+    dt_in = torch.full((T, R), -6.0)                         # steps of about 0.0025: a decay of 0.9975 a token
+    dt_in[5] = 3.0
+    zeros = torch.zeros(R)
+    want, _ = P.selective_scan(x[:, :inner].double().reshape(T, R, P_), x[:, inner:inner + N].double().reshape(T, 1, N),
+                               x[:, inner + N:].double().reshape(T, 1, N), P.softplus(dt_in.double()), zeros.double(),
+                               zeros.double())
+    assert want[-1].abs().min() > 100                        # the early token is still there
+    for cuts in ([T], [6] + [1] * (T - 6), [2] * (T // 2)):
+        state = torch.zeros(2, 4 * ops.ssm_state_floats(R, P_, N), dtype=torch.uint8, device="cuda")
+        rows, at = [], 0
+        for c in cuts:
+            y = torch.empty(c, inner, device="cuda")
+            ops.ssm_scan(y, dev(x[at:at + c].contiguous()), dev(dt_in[at:at + c].contiguous()), dev(zeros), dev(zeros),
+                         dev(zeros), state, 0, i32([0, c]), i32([1]), c, 1, R, Q, N, P_)
+            rows.append(y.cpu())
+            at += c
+        assert torch.allclose(torch.cat(rows).double(), want.reshape(T, inner), rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,W,parts", [(5, 48, 1), (3, 60, 3), (70, 1024, 2), (2, 2304, 4)])
+def test_gated_grouped_norm(ops, dtype, rows, W, parts):
+    tdt = TORCH[dtype]
+    y, z = rnd(rows, W, seed=1, scale=3.0), rnd(rows, W + 9, seed=2, scale=2.0).to(tdt)
+    weight = (1 + 0.3 * rnd(W, seed=3)).to(tdt)
+    out = torch.empty(rows, W, dtype=tdt, device="cuda")
+    ops.gated_group_norm(out, dev(y), dev(z)[:, 4:4 + W], dev(weight), rows, parts, 1e-5)
+    want = P.gated_group_norm(y.double(), z[:, 4:4 + W].double(), weight.double(), parts, 1e-5)
+    tol = 3e-6 if dtype == "float32" else 2 ** -7
+    assert torch.allclose(out.cpu().double(), want, rtol=tol, atol=tol)
+
+
+# ------------------------------------------------------------------ the router's choice
+def routed(ops, logits, corr, real, groups, keep, top, scale):
+    rows, E = logits.shape
+    dense = torch.empty(rows, real + 1, device="cuda")
+    ids = torch.empty(rows, top, dtype=torch.int32, device="cuda")
+    weights = torch.empty(rows, top, device="cuda")
+    ops.route_tokens(dense, ids, weights, dev(logits), None if corr is None else dev(corr), rows, real, groups, keep, top, scale)
+    return dense.cpu(), ids.cpu(), weights.cpu()
+
+
+@pytest.mark.parametrize("cdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("E,real,groups,keep,top", [(20, 16, 2, 1, 4), (12, 12, 4, 2, 3), (7, 3, 1, 1, 7), (130, 128, 10, 3, 8),
+                                                    (6, 5, 6, 6, 1), (9, 9, 3, 1, 3)])
+def test_choice_among_groups_equals_the_plain_one(ops, cdtype, E, real, groups, keep, top):
+    rows = 33
+    logits = rnd(rows, E, seed=E, scale=2.0)
+    corr = rnd(E, seed=E + 1, scale=0.3).to(cdtype)            # larger than most scores: numbers below zero are common
+    dense, ids, weights = routed(ops, logits, corr, real, groups, keep, top, 1.7)
+    r = {"top": top, "scale": 1.7, "groups": {"count": groups, "keep": keep}}
+    for t in range(rows):
+        want = P.route(logits[t].double(), corr.double(), r)
+        assert ids[t].tolist() == [e for e, _ in want]
+        assert torch.allclose(weights[t].double(), torch.tensor([w for _, w in want], dtype=torch.float64), rtol=1e-5, atol=1e-7)
+        row = torch.zeros(real + 1, dtype=torch.float64)
+        for e, w in want:
+            row[min(e, real)] += w
+        assert torch.allclose(dense[t].double(), row, rtol=1e-5, atol=1e-7)
+        assert (dense[t] != 0).sum().item() <= top
+
+
+def test_choice_stays_inside_the_kept_groups_when_every_number_is_negative(ops):
+    logits = torch.tensor([[0.0, 0.1, 3.0, 0.2, 0.0, 0.1]])
+    corr = torch.tensor([-5.0, -5.0, -9.0, -9.0, -1.0, -1.2])
+    dense, ids, weights = routed(ops, logits, corr, 5, 3, 1, 2, 2.0)
+    s = torch.softmax(logits[0].double(), 0)
+    assert ids[0].tolist() == [4, 5]                           # a mask of zeros would have let outputs 0 and 1 in
+    assert torch.allclose(weights[0].double(), 2.0 * s[[4, 5]], rtol=1e-6)
+    assert torch.allclose(dense[0].double(), torch.tensor([0, 0, 0, 0, 2.0 * s[4], 2.0 * s[5]], dtype=torch.float64), rtol=1e-6)
+    # no correction: the plain scores choose, the group of the best output first
+    dense, ids, _ = routed(ops, logits, None, 6, 3, 2, 3, 1.0)
+    assert ids[0].tolist() == [2, 3, 1]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,real,I,extra", [(5, 3, 16, 24), (70, 6, 40, 0), (2, 1, 7, 5)])
+def test_weighted_expert_activation(ops, dtype, rows, real, I, extra):
+    tdt = TORCH[dtype]
+    gu = rnd(rows, 2 * real * I, seed=1, scale=2.5).to(tdt)
+    h = rnd(rows, extra, seed=2).to(tdt) if extra else None
+    dense = rnd(rows, real + 1, seed=3).abs()
+    dense[:, 0] = 0                                            # an expert nobody chose
+    dense[0, -1] = 0
+    gu[:, :2 * I] = float("inf")                               # whatever its rows hold, its stretch is exact zeros
+    out = torch.empty(rows, real * I + extra, dtype=tdt, device="cuda")
+    ops.routed_act(out, dev(gu), dev(dense), None if h is None else dev(h), rows, real, I, alpha=1.702, limit=1.25, up_shift=1.0)
+    g = gu.double().reshape(rows, real * I, 2)
+    act = torch.clamp(g[..., 0], max=1.25)
+    act = act * torch.sigmoid(1.702 * act) * (torch.clamp(g[..., 1], -1.25, 1.25) + 1)
+    want = act * dense[:, :real].double().repeat_interleave(I, 1)
+    want[:, :I] = 0
+    if extra:
+        want = torch.cat([want, dense[:, -1:].double() * h.double()], 1)
+    tol = 3e-6 if dtype == "float32" else 2 ** -7
+    assert torch.allclose(out.cpu().double(), want, rtol=tol, atol=tol)
+
+
+# ------------------------------------------------------------------ differential heads, query temperature
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,hd,vd", [(4, 2, 64, 64), (6, 1, 48, 40), (3, 3, 16, 8), (2, 2, 128, 100)])
+def test_the_two_maps_of_a_head_are_joined(ops, dtype, H, G, hd, vd):
+    tdt = TORCH[dtype]
+    rows, R = 7, H // G
+    attn_out = rnd(rows, 2 * H, hd, seed=4).to(tdt)
+    lam, diff, eps = 0.37, 0.6, 1e-5
+    out = torch.empty(rows, H * vd, dtype=tdt, device="cuda")
+    ops.diff_heads(out, dev(attn_out), rows, H, G, hd, vd, lam, 1 - diff, eps)
+    a = attn_out.double()
+    want = torch.zeros(rows, H, vd, dtype=torch.float64)
+    for h in range(H):
+        g, r = divmod(h, R)
+        o = a[:, (2 * g) * R + r, :vd] - lam * a[:, (2 * g + 1) * R + r, :vd]
+        want[:, h] = P.rms(o, eps) * (1 - diff)
+    tol = 3e-6 if dtype == "float32" else 2 ** -7
+    assert torch.allclose(out.cpu().double().reshape(rows, H, vd), want, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("coef,every", [(0.5, 64), (1.0, 1), (0.3, 7)])
+def test_query_temperature_at_its_steps(ops, dtype, coef, every):
+    tdt = TORCH[dtype]
+    H, hd = 3, 16
+    positions = [0, every - 2, every - 1, every, 2 * every - 2, 2 * every - 1, 5000]
+    positions = [max(p, 0) for p in positions]
+    rows = len(positions)
+    q_in, bias = rnd(rows, H * hd, seed=1).to(tdt), rnd(H * hd, seed=2).to(tdt)
+    q_out = torch.empty(rows, H * hd, dtype=tdt, device="cuda")
+    ops.qkv_rope_cache(q_out, None, None, dev(q_in), H * hd, 0, dev(bias), i32(positions), i32([0] * rows), i32([0]), None,
+                       None, 0, rows, H, 0, hd, False, q_temp=(coef, every))
+    temps = torch.tensor([P.query_temperature(p, coef, every) for p in positions], dtype=torch.float64)
+    assert temps[0] == (1.0 if every > 1 else 1 + coef * math.log(2))
+    want = (q_in.double() + bias.double()) * temps[:, None]
+    tol = 3e-6 if dtype == "float32" else 2 ** -7
+    assert torch.allclose(q_out.cpu().double(), want, rtol=tol, atol=tol)
+
+
+# ------------------------------------------------------------------ whole models
+MODELS = {
+    # attention first; a group of two query heads, values wider than keys, a temperature that steps every 16
+    # positions; a scan whose state size is no multiple of its threads' share, one group, four taps; experts in four
+    # groups of which two are kept
+    "P1": {"architecture": "Penasun", "vocab": 211, "width": 48, "norm": {"eps": 1e-6},
+           "layers": [layer("attention", attn(4, 2, 16, 32, 0.25, 0.5, (0.3, 16)), moe(6, 2, 2, 40, 1.5, 4, 2, 1.0)),
+                      layer("mamba2", scan(3, 16, 20, 1, 4, 1), moe(6, 2, 2, 40, 1.5, 4, 2, 1.0)),
+                      layer("attention", attn(4, 2, 16, 32, 0.25, 0.5, (0.3, 16)))]},
+    # a scan first and without a feed-forward; a large state, as many groups as heads, two taps; as many kv heads
+    # as heads, keys wider than values, no temperature; one expert a token, no identity experts, one group; then a
+    # scan with as many identity experts as others, every group kept
+    "P2": {"architecture": "Penasun", "vocab": 130, "width": 64, "norm": {"eps": 1e-5},
+           "layers": [layer("mamba2", scan(4, 24, 96, 4, 2, 4)),
+                      layer("attention", attn(3, 3, 24, 8, 0.2, 0.8), moe(5, 0, 1, 24, 0.5, 1, 1, 2.5)),
+                      layer("mamba2", scan(2, 40, 16, 2, 3, 1), moe(4, 4, 3, 16, 7.0, 2, 2, 0.5))]},
+    # one kv head for six heads with head sizes that are no multiple of 16, a temperature that steps at every
+    # position; one kept group of three; a second attention of another shape; a scan with a single tap
+    "P3": {"architecture": "Penasun", "vocab": 97, "width": 40, "norm": {"eps": 1e-6},
+           "layers": [layer("attention", attn(6, 1, 8, 40, 0.35, 0.3, (1.0, 1)), moe(9, 3, 4, 32, 1.0, 3, 1, 1.5)),
+                      layer("attention", attn(2, 2, 32, 32, 0.18, 0.6, (0.5, 70)), moe(2, 0, 2, 56, 1.0)),
+                      layer("mamba2", scan(5, 8, 64, 1, 1, 5), moe(3, 1, 1, 24, 2.0, 2, 1, 1.0))]},
+}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    """name -> model folder. The q and k matrices are made larger than the random default so that the attention
+    weights are far from uniform and a key that is wrongly seen or missed matters; the other matrices so that
+    the experts' bounds bind; the corrections so that they, and not the scores, decide most choices."""
+    import hector_engine_amd  # noqa: F401
+    from hector_engine_amd.registry import config_from_dict
+    from hector_engine_amd.weights import write_random_model
+    from hector_engine_amd.weights.safetensors_io import write_safetensors
+    from safetensors.torch import load_file
+    out = {}
+    for i, (name, cfg) in enumerate(MODELS.items()):
+        for calm in (False, True):
+            folder = str(tmp_path_factory.mktemp(f"penasun_{name}"))
+            write_random_model(config_from_dict(json.loads(json.dumps(cfg))), 60 + i, folder, "bfloat16")
+            path = folder + "/model.safetensors"
+            tensors = load_file(path)
+            for k in tensors:
+                if k.endswith(".mix.q") or k.endswith(".mix.k"):
+                    tensors[k] = (tensors[k].float() * 12).to(torch.bfloat16)
+                elif k.endswith(".correction"):
+                    tensors[k] = (tensors[k].float() * 10).to(torch.bfloat16)
+                elif k.endswith(".mix.conv") or k == "embed" or (calm and k.endswith(".router")):
+                    pass
+                elif tensors[k].dim() == 2:
+                    tensors[k] = (tensors[k].float() * 4).to(torch.bfloat16)
+            write_safetensors(path, tensors, {"format": "pt"})
+            out[name + "_calm" if calm else name] = folder
+    return out
+
+
+def variant(name, dtype):
+    """The folder a precision is tested on. In 32-bit the routers' rows are as large as the other matrices, so
+    that the tokens of a request choose many different experts. Under bfloat16 a token whose two best choice
+    numbers lie within the rounding of the rows in front of the router takes another expert than the plain
+    implementation (with the plain bfloat16 kernels as with the fast ones: a sixth of the positions of such a
+    request is then off by 5 to 40 % of the logits' spread); there the routers' rows keep their small random
+    values, the scores of a token differ little and the corrections decide most choices."""
+    return name if dtype == "float32" else name + "_calm"
+
+
+@pytest.fixture(scope="module")
+def plain(folders):
+    return {name: P.read_model(f) for name, f in folders.items()}
+
+
+@pytest.fixture(scope="module")
+def engines(folders):
+    import hector_engine_amd as he
+    cache = {}
+
+    def get(name, dtype, **kw):
+        key = (name, dtype, tuple(sorted(kw.items())))
+        if key not in cache:
+            opts = dict(max_tokens=4096, max_slots=8, max_seq_len=1024)
+            opts.update(kw)
+            cache[key] = he.Engine(folders[variant(name, dtype)], dtype=dtype, **opts)
+        return cache[key]
+
+    return get
+
+
+def same(got, want, dtype):
+    """float32: every logit to a few ulp of the logits' size. bfloat16: a token whose two best choice numbers
+    lie closer than the rounding of the rows in front of the router takes another expert than the plain
+    implementation's, in the plain bfloat16 kernels as in the fast ones, and what follows it in the sequence
+    inherits some of that. So the bound is on the bulk of the positions: per position the root mean square of
+    the logits' error (mean taken off) against that of the logits; the median stays under 4 % and all but a
+    seventh of the positions (or one) under 8 %. Measured: medians of 0.7 to 2 %, 90 % of the positions under 1
+    to 4 %, single positions up to 38 %."""
+    if dtype == "float32":
+        return close(got, want, dtype)
+    got, want = got.detach().cpu().double(), want.double()
+    assert got.shape == want.shape
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    w = want - want.mean(-1, keepdim=True)
+    r = d.pow(2).mean(-1).sqrt() / w.pow(2).mean(-1).sqrt()
+    assert bool(torch.isfinite(r).all())
+    assert (r > 0.08).sum().item() <= max(1, len(r) // 7), r
+    if len(r) >= 8:
+        assert r.median().item() <= 0.04, r
+
+
+def entry(slot, tokens, want):
+    from hector_engine_amd.engine.engine import StepEntry
+    return StepEntry(slot, list(tokens), list(want))
+
+
+def test_the_folder_written_from_a_configuration_reads_back(folders):
+    from hector_engine_amd.registry import load_config
+    for name, folder in folders.items():
+        assert load_config(folder).to_dict() == json.load(open(folder + "/config.json")) == MODELS[name.split("_")[0]]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(MODELS))
+def test_each_request_alone_and_whole(engines, plain, name, dtype):
+    eng = engines(name, dtype)
+    cfg, w = plain[variant(name, dtype)]
+    for seed, n in enumerate([1, 2, 23, 64, 65, 150]):
+        ids = rand_ids(cfg["vocab"], n, seed)
+        s = eng.acquire()
+        got = eng.step([entry(s, ids, range(n))])
+        want = P.forward(cfg, w, ids)[0]
+        same(got, want, dtype)
+        if dtype == "float32":
+            argmax_agrees_where_clear(got, want, 0.05 * want.abs().max().item())
+        eng.release(s)
+
+
+@pytest.mark.parametrize("name", list(MODELS))
+def test_the_stream_after_every_layer(engines, plain, name):
+    eng = engines(name, "float32", use_graphs=False)
+    cfg, w = plain[name]
+    ids = rand_ids(cfg["vocab"], 70, 9)
+    want = []
+    P.forward(cfg, w, ids, None, want)
+    seen = []
+    originals = [b.forward for b in eng.model.blocks]
+    try:
+        for b, orig in zip(eng.model.blocks, originals):
+            def fwd(stream, ctx, cache, orig=orig):
+                orig(stream, ctx, cache)
+                seen.append(stream.materialize(ctx)[:ctx.rows].clone())
+            b.forward = fwd
+        s = eng.acquire()
+        eng.step([entry(s, ids, [69])])
+        eng.release(s)
+    finally:
+        for b, orig in zip(eng.model.blocks, originals):
+            b.forward = orig
+    assert len(seen) == len(want)
+    for got, ref in zip(seen, want):
+        assert torch.allclose(got.cpu().double(), ref, rtol=2e-5, atol=2e-5 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(MODELS))
+def test_prompt_then_token_by_token_over_page_edges(engines, plain, name, dtype):
+    eng = engines(name, dtype)
+    cfg, w = plain[variant(name, dtype)]
+    n, tail = 210, 150                  # the decoded positions 60..209 cross two page edges and every temperature step
+    ids = rand_ids(cfg["vocab"], n, 11)
+    want = P.forward(cfg, w, ids)[0]
+    s = eng.acquire()
+    whole = eng.step([entry(s, ids, range(n))]).clone()
+    eng.release(s)
+    s = eng.acquire()
+    assert eng.step([entry(s, ids[:n - tail], [])]) is None
+    dec = torch.cat([eng.step([entry(s, [t], [0])]).clone() for t in ids[n - tail:]])
+    eng.release(s)
+    same(dec, want[n - tail:], dtype)
+    if dtype == "float32":
+        assert torch.equal(dec, whole[n - tail:])        # the 32-bit path does not depend on the cut
+    else:
+        same(dec, whole[n - tail:].cpu(), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(MODELS))
+@pytest.mark.parametrize("cuts", [[2] * 40, [3, 2, 61, 17, 64, 2, 70], [1, 1, 2, 1, 25, 47, 48, 2], [128, 2, 2, 65]])
+def test_prompts_fed_in_portions(engines, plain, name, dtype, cuts):
+    eng = engines(name, dtype)
+    cfg, w = plain[variant(name, dtype)]
+    n = sum(cuts)
+    ids = rand_ids(cfg["vocab"], n, 12)
+    want = P.forward(cfg, w, ids)[0]
+    s = eng.acquire()
+    whole = eng.step([entry(s, ids, range(n))]).clone()
+    eng.release(s)
+    s = eng.acquire()
+    parts, at = [], 0
+    for c in cuts:
+        parts.append(eng.step([entry(s, ids[at:at + c], range(c))]).clone())
+        at += c
+    eng.release(s)
+    got = torch.cat(parts)
+    same(got, want, dtype)
+    if dtype == "float32":
+        assert torch.equal(got, whole)
+    else:
+        same(got, whole.cpu(), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(MODELS))
+def test_unequal_batches_equal_each_request_alone_and_slots_are_used_again(engines, plain, name, dtype):
+    eng = engines(name, dtype, max_slots=4)
+    cfg, w = plain[variant(name, dtype)]
+    free = eng.cache.free_pages
+    for round_no, lengths in enumerate([[1, 67, 140, 25], [90, 3, 49], [200, 2, 2, 64]]):
+        prompts = [rand_ids(cfg["vocab"], n, 20 * round_no + i) for i, n in enumerate(lengths)]
+        decode = 12
+        full = [p + rand_ids(cfg["vocab"], decode - i, 500 + i) for i, p in enumerate(prompts)]   # shorter ones end earlier
+        want = [P.forward(cfg, w, f)[0] for f in full]
+        slots = [eng.acquire() for _ in prompts]
+        got = [[] for _ in prompts]
+        logits = eng.step([entry(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])
+        for i in range(len(prompts)):
+            got[i].append(logits[i:i + 1].clone())
+        live = list(range(len(prompts)))
+        for t in range(decode):
+            live = [i for i in live if len(prompts[i]) + t < len(full[i])]
+            if not live:
+                break
+            logits = eng.step([entry(slots[i], [full[i][len(prompts[i]) + t]], [0]) for i in live])
+            for j, i in enumerate(live):
+                got[i].append(logits[j:j + 1].clone())
+        for i, s in enumerate(slots):
+            eng.release(s)          # the next round's requests take these slots, and their states, again
+            same(torch.cat(got[i]), want[i][len(prompts[i]) - 1:], dtype)
+    assert eng.cache.free_pages == free
+
+
+@pytest.mark.parametrize("name", list(MODELS))
+def test_a_mixed_step_of_a_prompt_and_decoding_requests(engines, plain, name):
+    eng = engines(name, "float32")
+    cfg, w = plain[name]
+    a, b = rand_ids(cfg["vocab"], 80, 30), rand_ids(cfg["vocab"], 37, 31)
+    sa, sb = eng.acquire(), eng.acquire()
+    eng.step([entry(sa, a[:79], [])])
+    got = eng.step([entry(sa, a[79:], [0]), entry(sb, b, range(37))])
+    same(got[:1], P.forward(cfg, w, a)[0][-1:], "float32")
+    same(got[1:], P.forward(cfg, w, b)[0], "float32")
+    eng.release(sa)
+    eng.release(sb)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_long_request_and_long_decoding(engines, plain, dtype):
+    eng = engines("P1", dtype)
+    cfg, w = plain[variant("P1", dtype)]
+    n = 700
+    ids = rand_ids(cfg["vocab"], n, 41)
+    want = P.forward(cfg, w, ids)[0]
+    s = eng.acquire()
+    got = [eng.step([entry(s, ids[:400], [0, 63, 64, 399])]).clone()]
+    got += [eng.step([entry(s, [t], [0])]).clone() for t in ids[400:]]
+    eng.release(s)
+    same(torch.cat(got), torch.cat([want[[0, 63, 64, 399]], want[400:]]), dtype)
+
+
+@pytest.mark.parametrize("name", list(MODELS))
+def test_greedy_generation_through_the_library(folders, plain, name):
+    import hector_engine_amd as he
+    cfg, w = plain[name]
+    prompts = [rand_ids(cfg["vocab"], n, 70 + i) for i, n in enumerate([5, 30, 61])]
+    steps = 40
+    want = [P.greedy(cfg, w, p, steps) for p in prompts]
+    eng = he.Engine(folders[name], dtype="float32", max_tokens=2048, max_seq_len=512)
+    got = he.generate(eng, prompts, max_new_tokens=steps, stop_ids=())
+    assert [r.tokens for r in got] == want
+    small = he.Engine(folders[name], dtype="float32", max_tokens=2048, max_slots=2, max_seq_len=512)
+    assert [r.tokens for r in he.generate(small, prompts, max_new_tokens=steps, stop_ids=())] == want
+    assert small.cache.free_pages == small.cache.num_pages
+    cfg, w = plain[name + "_calm"]
+    want = [P.greedy(cfg, w, p, steps) for p in prompts]
+    eng16 = he.Engine(folders[name + "_calm"], dtype="bfloat16", max_tokens=2048, max_seq_len=512)
+    for p, r, t in zip(prompts, he.generate(eng16, prompts, max_new_tokens=steps, stop_ids=()), want):
+        seq = list(p)
+        for x, y in zip(r.tokens, t):
+            if x != y:
+                top = P.forward(cfg, w, seq)[0][-1].topk(2).values
+                assert (top[0] - top[1]).item() < 0.03 * top[0].abs().item() + 1e-3      # a near tie
+                break
+            seq.append(x)
+
+
+def test_the_command_line_and_the_trace_replay_serve_it(folders, plain, tmp_path):
+    import numpy as np
+    from tests.conftest import ROOT
+    cfg, w = plain["P2"]
+    exe = os.path.join(ROOT, "bin", "hector_generate")
+    out = subprocess.run([sys.executable, exe, folders["P2"], "5,17,3;9,2,77,13", "6", "--dtype", "float32",
+                          "--stop-ids", ""], capture_output=True, text=True, timeout=180)
+    assert out.returncode == 0, out.stderr
+    for i, p in enumerate(([5, 17, 3], [9, 2, 77, 13])):
+        assert f"[{i}] prompt" in out.stdout and ",".join(map(str, P.greedy(cfg, w, p, 6))) in out.stdout
+    assert "Penasun" in out.stdout
+    reqs = {"a": rand_ids(cfg["vocab"], 4, 1), "b": rand_ids(cfg["vocab"], 68, 2), "c": rand_ids(cfg["vocab"], 133, 3)}
+    steps = [{"step": 0, "entries": [{"id": k, "tokens": v[:-3], "want": [len(v) - 4]} for k, v in reqs.items()], "end": []}]
+    for t in range(3):
+        steps.append({"step": t + 1, "entries": [{"id": k, "tokens": [v[len(v) - 3 + t]], "want": [0]} for k, v in reqs.items()],
+                      "end": list(reqs) if t == 2 else []})
+    for dtype in DTYPES:
+        out_dir = str(tmp_path / dtype)
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders["P2"],
+                               "--dtype", dtype, "--out", out_dir, "--max-tokens", "196"],
+                              input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=180)
+        assert proc.returncode == 0, proc.stderr
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+        want = {k: P.forward(cfg, w, v)[0] for k, v in reqs.items()}
+        for s in range(4):
+            got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{s}.f32"), dtype="<f4").reshape(3, -1).copy())
+            rows = torch.stack([want[k][len(reqs[k]) - 4 + s] for k in reqs])
+            same(got, rows, dtype)
