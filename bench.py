@@ -4,7 +4,7 @@ token ids) on one MI355X, with prefill and roofline figures on the same line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b|32b|72b]
                     [--context C] [--prompt P]
-    python bench.py --design volonex      (another measurement: see below)
+    python bench.py --design volonex | penasun      (another measurement: see below)
 
 The default is the 7B shape; --shape runs the same measurement at the layer sizes of
 Qwen2.5-32B (context 8192, prompts of 512 to 2048 tokens, batches 1 / 8 / 64) or
@@ -28,7 +28,7 @@ the machine runs every kernel of the one-token step 4 to 6 % slower than afterwa
 leaves its first run and its thermal-low samples out: OPTIMIZATION_NOTES.md:114-117); `repeats` holds
 every timed run, the earlier ones still show it.
 
---design volonex leaves the run above aside and measures the Volonex design beside Qwen2 at equal layer
+--design volonex (or penasun) leaves the run above aside and measures that design beside Qwen2 at equal layer
 sizes (random weights, bf16, four layers of each of a few sizes that resemble real models' layers): prompt
 tokens a second for one prompt of 2,048 tokens, decoded tokens a second at batch 8 and batch 1 behind such
 prompts, and, from a second pass with an event pair around every launch, the mean time of each kind of
@@ -121,6 +121,24 @@ def design_configs(sz):
     return config_from_dict(qwen), config_from_dict(volonex)
 
 
+def penasun_configs(sz):
+    """(Qwen2 configuration, Penasun configuration) of one set of layer sizes: state-space and differential
+    attention layers in turn (the scan's inner width twice the model's, heads of 64, a state of 128; two score maps
+    of half the Qwen2 head's width each), every layer with 16 experts and 2 identity experts of which a token
+    uses 4, each a quarter of the Qwen2 feed-forward wide: a token's own arithmetic is that of the Qwen2 layer."""
+    from hector_engine_amd.registry import config_from_dict
+    qwen, _ = design_configs(sz)
+    scan = dict(type="mamba2", mixer=dict(heads=2 * sz["width"] // 64, vdim=64, state=128, groups=8, conv=4, norm_groups=8))
+    attention = dict(type="attention", mixer=dict(heads=sz["heads"], kv_heads=sz["kv_heads"], dim=sz["dim"] // 2,
+                                                  vdim=sz["vdim"], scale=(sz["dim"] // 2) ** -0.5, diff=0.6,
+                                                  q_temp=dict(coef=0.1, every=512)))
+    mlp = dict(kind="moe", expert=dict(ff=sz["ff"] // 4, limit=7.0),
+               router=dict(experts=16, identity=2, top=4, scale=1.0, groups=dict(count=3, keep=2)))
+    layers = [dict(l, mlp=mlp) for l in (scan, attention)] * (DESIGN_LAYERS // 2)
+    penasun = dict(architecture="Penasun", vocab=DESIGN_VOCAB, width=sz["width"], norm=dict(eps=1e-6), layers=layers)
+    return qwen, config_from_dict(penasun)
+
+
 def compare_designs(args) -> int:
     import torch
     import hector_engine_amd as he
@@ -199,13 +217,16 @@ def compare_designs(args) -> int:
         return out
 
     result = {}
-    for name, sz in DESIGN_SIZES.items():
+    chosen = [n for n in DESIGN_SIZES if not args.design_sizes or n in args.design_sizes.split(",")]
+    for name in chosen:
+        sz = DESIGN_SIZES[name]
         result[name] = {"sizes": sz}
-        for design, config in zip(("qwen2", "volonex"), design_configs(sz)):
+        configs = design_configs(sz) if args.design == "volonex" else penasun_configs(sz)
+        for design, config in zip(("qwen2", args.design), configs):
             progress(f"{name} {design}")
             result[name][design] = measure(config, False)
             result[name][design].update(measure(config, True))
-    print(json.dumps({"metric": "design_comparison", "design": "volonex", "beside": "qwen2", "dtype": "bf16",
+    print(json.dumps({"metric": "design_comparison", "design": args.design, "beside": "qwen2", "dtype": "bf16",
                       "data": "synthetic", "layers": DESIGN_LAYERS, "vocab": DESIGN_VOCAB, "prompt": prompt_len,
                       "batch": batch, "steps": steps, "sizes": result}))
     return 0
@@ -240,7 +261,8 @@ def main() -> int:
                     help="float32: the whole measurement in true 32-bit (no library products, no extra points)")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
-    ap.add_argument("--design", choices=["volonex"], default=None,
+    ap.add_argument("--design-sizes", default="", help=f"with --design: only these of {', '.join(DESIGN_SIZES)}")
+    ap.add_argument("--design", choices=["volonex", "penasun"], default=None,
                     help="instead of the run above: this design beside Qwen2 at equal layer sizes, prompt and "
                          "one-token steps, throughput and mean time per kind of kernel")
     args = ap.parse_args()
