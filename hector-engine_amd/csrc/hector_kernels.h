@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 22
+#define HE_ABI_VERSION 24
 
 #ifdef __cplusplus
 extern "C" {
@@ -221,17 +221,19 @@ int he_conv_state(void* out, const void* x, int64_t x_stride, const void* taps, 
                   int dtype, void* stream);
 int64_t he_ssm_state_floats(int R, int P, int N);
 // xbc [rows][R P + 2 Q N]: x, then the Q groups' B vectors, then their C vectors; dt_in[row * dt_stride + r].
-// y [rows][R P] fp32 (rows without a sequence are not written).
+// y [rows][R P] fp32 (rows without a sequence are not written). max_q_len: a bound on the rows a sequence brings (0: none).
 int he_ssm_scan(void* y_f32, const void* xbc, const void* dt_in, int64_t dt_stride, const void* dt_bias,
                 const void* a_log, const void* d_skip, int w_dtype, void* state, int64_t state_stride,
                 int64_t state_offset, const void* cu_seqlens, const void* seq_slot, int rows, int num_seqs,
-                int R, int Q, int N, int P, int dtype, void* stream);
+                int max_q_len, int R, int Q, int N, int P, int dtype, void* stream);
 // out = rms over each of `parts` stretches of (y * silu(z)) * weight; z[row * z_stride + c].
 int he_gated_group_norm(void* out, const void* y_f32, const void* z, int64_t z_stride, const void* weight,
                         int w_dtype, int rows, int W, int parts, float eps, int dtype, void* stream);
 
 // ---- routing and head combination (routing.hip) ---------------------------------
+// logits_f32 [rows][E], or null and x [rows][D] (x_dtype) with router_f32 [E][D]: the kernel forms the logits itself.
 int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32, const void* logits_f32,
+                    const void* x, int x_dtype, const void* router_f32, int D,
                     const void* correction, int c_dtype, int rows, int E, int real, int groups, int keep,
                     int top, float scale, void* stream);
 int he_routed_act(void* out, const void* gate_up, const void* dense_f32, const void* h, int rows, int real,

@@ -17,84 +17,144 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
   }
 }
 
-// One wavefront a row. logits [rows][E] fp32. s = softmax(logits) over all E outputs; the choice is made
+// One wavefront a row. logits [rows][E] fp32, or, with x and router given, the router's product itself:
+// logits[e] = sum_i x[row][i] * router[e][i] in fp32 (router fp32 [E][D]; a lane adds its elements i = lane,
+// lane + 64, ... in that order, the lanes' sums meet in the wavefront's butterfly: one fixed order a row,
+// whatever else the step holds). s = softmax(logits) over all E outputs; the choice is made
 // on c = s + correction: the E outputs form `groups` equal groups of neighbours, a group counts by its
 // largest c, only the outputs of the `keep` best groups can be chosen (the others count as -inf), and
 // the `top` largest c among those are chosen. The weight of a chosen output is s * scale (not c, and
 // not renormalised). The last E - real outputs are experts without weights whose result is the input
 // itself: their weights are added up in column `real` of dense. dense [rows][real + 1] holds the
 // weight of every expert (0 where not chosen); ids / weights [rows][top] list the chosen ones.
-__global__ __launch_bounds__(64) void route_kernel(float* __restrict__ dense, int32_t* __restrict__ ids,
-                                                   float* __restrict__ weights, const float* __restrict__ logits,
-                                                   const void* __restrict__ correction, int c_dtype, int E, int real,
-                                                   int groups, int keep, int top, float scale) {
+#define ROUTE_WAVES 8
+__global__ __launch_bounds__(64 * ROUTE_WAVES) void route_kernel(
+    float* __restrict__ dense, int32_t* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ logits,
+    const void* __restrict__ x, int x_dtype, const float* __restrict__ router, int D,
+    const void* __restrict__ correction, int c_dtype, int E, int real, int groups, int keep, int top, float scale) {
   __shared__ float s_sh[ROUTE_MAX_EXPERTS];
   __shared__ float c_sh[ROUTE_MAX_EXPERTS];
   __shared__ float d_sh[ROUTE_MAX_EXPERTS + 1];
   __shared__ float g_sh[ROUTE_MAX_EXPERTS];
+  __shared__ float z[ROUTE_MAX_EXPERTS];
   const int64_t row = blockIdx.x;
-  const int lane = threadIdx.x;
-  const float* z = logits + row * E;
-  float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
-  mx = wave_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += 64) {
-    const float v = expf(z[e] - mx);
-    s_sh[e] = v;
-    sum += v;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  // The first wavefront makes the choice; with x given, all of them form the logits first, each the outputs
+  // e = wave, wave + 8, ...: four elements a lane and turn, four sums a lane that meet in index order.
+  const bool lead = wave == 0;
+  if (x != nullptr) {
+    const bool vec = (D & 3) == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)router & 15) == 0;
+    for (int e = wave; e < E; e += ROUTE_WAVES) {
+      const float* w = router + (int64_t)e * D;
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      if (vec && x_dtype == HE_BF16) {
+        const uint2* xr = reinterpret_cast<const uint2*>((const uint16_t*)x + row * D);
+#pragma unroll 4
+        for (int i = lane; i < (D >> 2); i += 64) {
+          const uint2 xv = xr[i];
+          const float4 wv = reinterpret_cast<const float4*>(w)[i];
+          a0 = fmaf(__uint_as_float(xv.x << 16), wv.x, a0);
+          a1 = fmaf(__uint_as_float(xv.x & 0xffff0000u), wv.y, a1);
+          a2 = fmaf(__uint_as_float(xv.y << 16), wv.z, a2);
+          a3 = fmaf(__uint_as_float(xv.y & 0xffff0000u), wv.w, a3);
+        }
+      } else if (vec) {
+        const float4* xr = reinterpret_cast<const float4*>((const float*)x + row * D);
+#pragma unroll 4
+        for (int i = lane; i < (D >> 2); i += 64) {
+          const float4 xv = xr[i];
+          const float4 wv = reinterpret_cast<const float4*>(w)[i];
+          a0 = fmaf(xv.x, wv.x, a0);
+          a1 = fmaf(xv.y, wv.y, a1);
+          a2 = fmaf(xv.z, wv.z, a2);
+          a3 = fmaf(xv.w, wv.w, a3);
+        }
+      } else {
+        for (int i = lane; i < D; i += 64) {
+          const float xv = x_dtype == HE_BF16 ? bf16_bits_to_float(((const uint16_t*)x)[row * D + i])
+                                              : ((const float*)x)[row * D + i];
+          a0 = fmaf(xv, w[i], a0);
+        }
+      }
+      const float acc = wave_sum((a0 + a1) + (a2 + a3));
+      if (lane == 0) z[e] = acc;
+    }
+  } else if (lead) {
+    for (int e = lane; e < E; e += 64) z[e] = logits[row * E + e];
   }
-  sum = wave_sum(sum);
-  const float inv = 1.f / sum;
-  for (int e = lane; e < E; e += 64) {
-    const float s = s_sh[e] * inv;
-    s_sh[e] = s;
-    c_sh[e] = s + (correction ? load_param(correction, e, c_dtype) : 0.f);
+  __syncthreads();
+  // from here on the first wavefront works; the others only keep the barriers' count
+  if (lead) {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+      const float v = expf(z[e] - mx);
+      s_sh[e] = v;
+      sum += v;
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.f / sum;
+    for (int e = lane; e < E; e += 64) {
+      const float s = s_sh[e] * inv;
+      s_sh[e] = s;
+      c_sh[e] = s + (correction ? load_param(correction, e, c_dtype) : 0.f);
+    }
+    for (int e = lane; e <= real; e += 64) d_sh[e] = 0.f;
   }
-  for (int e = lane; e <= real; e += 64) d_sh[e] = 0.f;
   __syncthreads();
   const int size = E / groups;
   if (keep < groups) {
-    for (int g = lane; g < groups; g += 64) {
-      float best = -INFINITY;
-      for (int i = 0; i < size; ++i) best = fmaxf(best, c_sh[g * size + i]);
-      g_sh[g] = best;
+    if (lead) {
+      for (int g = lane; g < groups; g += 64) {
+        float best = -INFINITY;
+        for (int i = 0; i < size; ++i) best = fmaxf(best, c_sh[g * size + i]);
+        g_sh[g] = best;
+      }
     }
     __syncthreads();
     // the `keep` best groups are marked by +inf in g_sh, then the others' outputs are masked
     for (int k = 0; k < keep; ++k) {
       float v = -INFINITY;
       int idx = 0x7fffffff;
-      for (int g = lane; g < groups; g += 64) {
-        const float gv = g_sh[g];
-        if (gv != INFINITY && (gv > v || (gv == v && g < idx))) {
-          v = gv;
-          idx = g;
+      if (lead) {
+        for (int g = lane; g < groups; g += 64) {
+          const float gv = g_sh[g];
+          if (gv != INFINITY && (gv > v || (gv == v && g < idx))) {
+            v = gv;
+            idx = g;
+          }
         }
+        wave_argmax(v, idx);
       }
-      wave_argmax(v, idx);
       __syncthreads();
-      if (lane == 0 && idx < groups) g_sh[idx] = INFINITY;
+      if (lead && lane == 0 && idx < groups) g_sh[idx] = INFINITY;
       __syncthreads();
     }
-    for (int e = lane; e < E; e += 64)
-      if (g_sh[e / size] != INFINITY) c_sh[e] = -INFINITY;
+    if (lead) {
+      for (int e = lane; e < E; e += 64)
+        if (g_sh[e / size] != INFINITY) c_sh[e] = -INFINITY;
+    }
     __syncthreads();
   }
   for (int k = 0; k < top; ++k) {
     float v = -INFINITY;
     int idx = 0x7fffffff;
-    for (int e = lane; e < E; e += 64) {
-      const float cv = c_sh[e];
-      // a chosen output is marked by NaN, which no comparison takes
-      if (cv > v || (cv == v && e < idx)) {
-        v = cv;
-        idx = e;
+    if (lead) {
+      for (int e = lane; e < E; e += 64) {
+        const float cv = c_sh[e];
+        // a chosen output is marked by NaN, which no comparison takes
+        if (cv > v || (cv == v && e < idx)) {
+          v = cv;
+          idx = e;
+        }
       }
+      wave_argmax(v, idx);
     }
-    wave_argmax(v, idx);
     __syncthreads();
-    if (lane == 0) {
+    if (lead && lane == 0) {
       const bool found = idx < E;
       const int e = found ? idx : 0;
       const float w = found ? s_sh[e] * scale : 0.f;
@@ -107,12 +167,18 @@ __global__ __launch_bounds__(64) void route_kernel(float* __restrict__ dense, in
     }
     __syncthreads();
   }
-  for (int e = lane; e <= real; e += 64) dense[row * (real + 1) + e] = d_sh[e];
+  if (lead) {
+    for (int e = lane; e <= real; e += 64) dense[row * (real + 1) + e] = d_sh[e];
+  }
 }
 
 extern "C" int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32, const void* logits_f32,
+                               const void* x, int x_dtype, const void* router_f32, int D,
                                const void* correction, int c_dtype, int rows, int E, int real, int groups, int keep,
                                int top, float scale, void* stream) {
+  HE_REQUIRE((logits_f32 != nullptr) != (x != nullptr), "he_route_tokens: give the logits, or the rows and the router");
+  HE_REQUIRE(x == nullptr || (router_f32 != nullptr && D > 0 && (x_dtype == HE_BF16 || x_dtype == HE_F32)),
+             "he_route_tokens: the router's matrix is missing");
   HE_REQUIRE(rows >= 0 && E > 0 && E <= ROUTE_MAX_EXPERTS && real >= 0 && real <= E,
              "he_route_tokens: bad sizes E=%d real=%d (at most %d outputs)", E, real, ROUTE_MAX_EXPERTS);
   HE_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups,
@@ -120,9 +186,9 @@ extern "C" int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32
   HE_REQUIRE(top > 0 && top <= keep * (E / groups), "he_route_tokens: %d chosen of %d kept outputs", top,
              keep * (E / groups));
   if (rows == 0) return 0;
-  route_kernel<<<rows, 64, 0, (hipStream_t)stream>>>((float*)dense_f32, (int32_t*)ids_i32, (float*)weights_f32,
-                                                     (const float*)logits_f32, correction, c_dtype, E, real, groups,
-                                                     keep, top, scale);
+  route_kernel<<<rows, 64 * ROUTE_WAVES, 0, (hipStream_t)stream>>>((float*)dense_f32, (int32_t*)ids_i32, (float*)weights_f32,
+                                                     (const float*)logits_f32, x, x_dtype, (const float*)router_f32, D,
+                                                     correction, c_dtype, E, real, groups, keep, top, scale);
   return he_check_launch("he_route_tokens");
 }
 

@@ -1,8 +1,8 @@
 // Kernels of a state-space mixer (a selective scan with a short causal convolution in front and a
 // gated, grouped RMS norm behind), over the packed rows of a step. What a sequence carries from step
 // to step lives in its row of the cache's state area, in fp32: the last K-1 inputs of the
-// convolution, [K-1][C], and then the state of the scan, [R][P][Npad] (head, value dim, state dim
-// padded to the threads' share). Everything that enters the recurrence is fp32.
+// convolution, [K-1][C], and then the state of the scan, he_ssm_state_floats() floats in the order the
+// scan's threads hold them. Everything that enters the recurrence is fp32.
 #include "common.h"
 #include "hector_kernels.h"
 
@@ -114,13 +114,24 @@ extern "C" int he_conv_state(void* out, const void* x, int64_t x_stride, const v
 // with S [N][P] carried in fp32. A thread holds NPT neighbouring state dims of one value dim p; the NG
 // threads of a p are neighbouring lanes, and their partial sums of y meet in a butterfly whose order
 // does not depend on the step. A workgroup takes PB value dims of one (sequence, head) and walks the
-// sequence's rows in order.
-static inline int ss_npt(int N) { return N <= 64 ? 8 : 16; }
+// sequence's rows in order; what a token brings (its B and C, the x of the workgroup's value dims,
+// its step size and decay, which one thread a token computes) is staged through LDS a tile of tokens
+// at a time, the next tile's loads in flight while this one is computed. In the state area the
+// workgroup's share of S lies in the order its threads load it, 16 bytes a lane: [i / 4][thread][i % 4].
+#define SS_PRE 16      // values a thread fetches for the next tile
+// state dims a thread holds. Measured at 64 heads of 64 with a state of 128, one prompt of 2,048 tokens: 0.93 ms
+// with 8 (a wavefront a SIMD), 1.20 ms with 4 (two a SIMD, but every workgroup stages all of B and C for half as
+// many value dims)
+static inline int ss_npt(int N) { return N <= 512 ? 8 : 16; }
 static inline int ss_groups(int N) {
   const int npt = ss_npt(N);
   int ng = 1;
   while (ng * npt < N) ng *= 2;
   return ng;
+}
+static inline int ss_pb(int N, int P) {
+  const int most = 256 / ss_groups(N);
+  return P < most ? P : most;
 }
 
 template <typename T, int NPT>
@@ -128,64 +139,151 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
     float* __restrict__ y, const T* __restrict__ xbc, const T* __restrict__ dt_in, int64_t dt_stride,
     const void* __restrict__ dt_bias, const void* __restrict__ a_log, const void* __restrict__ d_skip, int w_dtype,
     uint8_t* __restrict__ state, int64_t state_stride, int64_t state_offset, const int32_t* __restrict__ cu_seqlens,
-    const int32_t* __restrict__ seq_slot, int R, int Q, int N, int P, int NG, int PB) {
+    const int32_t* __restrict__ seq_slot, int R, int Q, int N, int P, int NG, int PB, int TT) {
+  extern __shared__ float4 ss_lds4[];
+  float* lds = reinterpret_cast<float*>(ss_lds4);
   const int seq = blockIdx.z, r = blockIdx.y;
   const int slot = seq_slot[seq];
   if (slot < 0) return;
   const int t0 = cu_seqlens[seq], t1 = cu_seqlens[seq + 1];
   if (t1 <= t0) return;
-  const int ng = threadIdx.x % NG;
-  const int p_raw = blockIdx.x * PB + threadIdx.x / NG;
-  const bool live = p_raw < P;
-  const int p = live ? p_raw : P - 1;
+  const int tid = threadIdx.x, threads = blockDim.x;
+  const int ng = tid % NG;
+  const bool own = tid < PB * NG;                       // the thread holds a share of the state
+  const int pl = own ? tid / NG : 0;
+  const int p0 = blockIdx.x * PB;
+  const bool live = own && p0 + pl < P;
   const int n0 = ng * NPT;
   const int Npad = NG * NPT;
+  const int W = (2 * Npad + PB + 2 + 3) & ~3;           // floats a token takes in LDS: B, C, x, dt, decay
   const int inner = R * P;
   const int C = inner + 2 * Q * N;
   const int q = r / (R / Q);
+  const int share = PB * NG * NPT;                      // floats of the workgroup's part of S
   float* S = reinterpret_cast<float*>(state + (int64_t)slot * state_stride + state_offset) +
-             ((int64_t)r * P + p) * Npad + n0;
+             ((int64_t)r * gridDim.x + blockIdx.x) * share;
   float s[NPT];
 #pragma unroll
-  for (int i = 0; i < NPT; ++i) s[i] = S[i];
+  for (int i4 = 0; i4 < NPT / 4; ++i4) {
+    const float4 v = own ? *reinterpret_cast<const float4*>(S + ((int64_t)i4 * PB * NG + tid) * 4) : make_float4(0, 0, 0, 0);
+    s[4 * i4] = v.x, s[4 * i4 + 1] = v.y, s[4 * i4 + 2] = v.z, s[4 * i4 + 3] = v.w;
+  }
   const float a = -expf(load_param(a_log, r, w_dtype));
   const float dk = load_param(d_skip, r, w_dtype);
   const float db = load_param(dt_bias, r, w_dtype);
-  for (int t = t0; t < t1; ++t) {
-    const T* row = xbc + (int64_t)t * C;
-    const float x = to_float(row[r * P + p]);
-    const float dt = ss_softplus(to_float(dt_in[(int64_t)t * dt_stride + r]) + db);
-    const float decay = expf(a * dt);
-    const float dtx = dt * x;
-    const T* Bv = row + inner + q * N;
-    const T* Cv = Bv + Q * N;
-    float acc = 0.f;
+  const int tile_floats = TT * W;
+  // What thread `tid` stages of a tile does not change from tile to tile: value k is token tt_k's float j_k,
+  // which comes from column col_k of the token's row of xbc (B, C, x) or of dt_in (step size, decay), or is
+  // padding. The loads carry no branch (a padding value reads column 0 and is dropped), so that a tile's loads
+  // go out together and stay in flight while the tile before is computed; they are turned into values,
+  // softplus and decay included, when they are written to LDS.
+  enum { SS_ZERO = 0, SS_VALUE = 1, SS_DT = 2, SS_DECAY = 3 };
+  int col[SS_PRE], tok_of[SS_PRE];
+  unsigned kinds = 0;                                  // two bits a value
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) {
-      const int n = n0 + i;
-      const float b = n < N ? to_float(Bv[n]) : 0.f;
-      const float c = n < N ? to_float(Cv[n]) : 0.f;
-      s[i] = fmaf(decay, s[i], dtx * b);
-      acc = fmaf(s[i], c, acc);
+  for (int k = 0; k < SS_PRE; ++k) {
+    col[k] = 0, tok_of[k] = 0;
+    if (k * threads >= tile_floats) break;             // (a one-token step stages a few hundred values, not thousands)
+    const int idx = tid + k * threads;
+    const int tt = idx / W, j = idx - tt * W;
+    int kind = SS_ZERO, c = 0;
+    if (idx < tile_floats) {
+      if (j < Npad) {
+        if (j < N) kind = SS_VALUE, c = inner + q * N + j;
+      } else if (j < 2 * Npad) {
+        if (j - Npad < N) kind = SS_VALUE, c = inner + (Q + q) * N + (j - Npad);
+      } else if (j < 2 * Npad + PB) {
+        if (p0 + (j - 2 * Npad) < P) kind = SS_VALUE, c = r * P + p0 + (j - 2 * Npad);
+      } else if (j < 2 * Npad + PB + 2) {
+        kind = j == 2 * Npad + PB ? SS_DT : SS_DECAY, c = r;
+      }
     }
-    for (int m = 1; m < NG; m <<= 1) acc += __shfl_xor(acc, m);
-    if (ng == 0 && live) y[(int64_t)t * inner + r * P + p] = fmaf(dk, x, acc);
+    col[k] = c;
+    tok_of[k] = tt;
+    kinds |= (unsigned)kind << (2 * k);
   }
-  if (live) {
+  T pre[SS_PRE];
+  auto fetch = [&](int first) {
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) S[i] = s[i];
+    for (int k = 0; k < SS_PRE; ++k) {
+      if (k * threads >= tile_floats) break;           // (the same for the whole workgroup)
+      const int kind = (kinds >> (2 * k)) & 3;
+      const int t = min(first + tok_of[k], t1 - 1);
+      const T* src = kind >= SS_DT ? dt_in + (int64_t)t * dt_stride : xbc + (int64_t)t * C;
+      pre[k] = src[col[k]];
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int k = 0; k < SS_PRE; ++k) {
+      if (k * threads >= tile_floats) break;
+      const int idx = tid + k * threads;
+      const int kind = (kinds >> (2 * k)) & 3;
+      float v = kind == SS_ZERO ? 0.f : to_float(pre[k]);
+      if (kind >= SS_DT) {
+        const float dt = ss_softplus(v + db);
+        v = kind == SS_DT ? dt : expf(a * dt);
+      }
+      if (idx < tile_floats) lds[buf * tile_floats + idx] = v;
+    }
+  };
+  fetch(t0);
+  put(0);
+  __syncthreads();
+  int buf = 0;
+  for (int first = t0; first < t1; first += TT, buf ^= 1) {
+    const bool more = first + TT < t1;
+    if (more) fetch(first + TT);
+    const int count = min(TT, t1 - first);
+    for (int tt = 0; tt < count; ++tt) {
+      const float* tok = lds + buf * tile_floats + tt * W;
+      const float x = tok[2 * Npad + pl];
+      const float dt = tok[2 * Npad + PB];
+      const float decay = tok[2 * Npad + PB + 1];
+      const float dtx = dt * x;
+      float acc = 0.f;
+#pragma unroll
+      for (int i4 = 0; i4 < NPT / 4; ++i4) {
+        const float4 b4 = *reinterpret_cast<const float4*>(tok + n0 + 4 * i4);
+        const float4 c4 = *reinterpret_cast<const float4*>(tok + Npad + n0 + 4 * i4);
+        const float b[4] = {b4.x, b4.y, b4.z, b4.w}, c[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s[4 * i4 + e] = fmaf(decay, s[4 * i4 + e], dtx * b[e]);
+          acc = fmaf(s[4 * i4 + e], c[e], acc);
+        }
+      }
+      // the NG neighbouring lanes of a value dim: through the vector ALU's own lane exchanges (every lane
+      // of the wavefront runs this loop, which they require)
+      if (NG > 1) acc += lane_xor1(acc);
+      if (NG > 2) acc += lane_xor2(acc);
+      if (NG > 4) acc += lane_xor4(acc);
+      if (NG > 8) acc += lane_xor8(acc);
+      if (NG > 16) acc = xor16_sum(acc);
+      if (NG > 32) acc = xor32_sum(acc);
+      if (ng == 0 && live) y[(int64_t)(first + tt) * inner + r * P + p0 + pl] = fmaf(dk, x, acc);
+    }
+    if (more) put(buf ^ 1);
+    __syncthreads();
+  }
+  if (own) {
+#pragma unroll
+    for (int i4 = 0; i4 < NPT / 4; ++i4)
+      *reinterpret_cast<float4*>(S + ((int64_t)i4 * PB * NG + tid) * 4) =
+          make_float4(s[4 * i4], s[4 * i4 + 1], s[4 * i4 + 2], s[4 * i4 + 3]);
   }
 }
 
 extern "C" int64_t he_ssm_state_floats(int R, int P, int N) {
   if (R <= 0 || P <= 0 || N <= 0) return 0;
-  return (int64_t)R * P * ss_groups(N) * ss_npt(N);
+  const int PB = ss_pb(N, P);
+  return (int64_t)R * ((P + PB - 1) / PB) * PB * ss_groups(N) * ss_npt(N);
 }
 
 extern "C" int he_ssm_scan(void* y_f32, const void* xbc, const void* dt_in, int64_t dt_stride, const void* dt_bias,
                            const void* a_log, const void* d_skip, int w_dtype, void* state, int64_t state_stride,
                            int64_t state_offset, const void* cu_seqlens, const void* seq_slot, int rows, int num_seqs,
-                           int R, int Q, int N, int P, int dtype, void* stream) {
+                           int max_q_len, int R, int Q, int N, int P, int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && num_seqs >= 0 && R > 0 && Q > 0 && N > 0 && P > 0 && R % Q == 0,
              "he_ssm_scan: bad sizes R=%d Q=%d N=%d P=%d", R, Q, N, P);
   HE_REQUIRE(N <= 1024, "he_ssm_scan: state size %d above 1024", N);
@@ -195,18 +293,25 @@ extern "C" int he_ssm_scan(void* y_f32, const void* xbc, const void* dt_in, int6
              "he_ssm_scan: the state row is too short or not aligned");
   if (rows == 0 || num_seqs == 0) return 0;
   const int NG = ss_groups(N);
-  const int PB = 256 / NG < P ? 256 / NG : P;
+  const int PB = ss_pb(N, P);
   const int threads = (PB * NG + 63) / 64 * 64;
+  const int W = (2 * NG * ss_npt(N) + PB + 2 + 3) & ~3;
+  int TT = SS_PRE * threads / W;
+  TT = TT < 1 ? 1 : (TT > 16 ? 16 : TT);
+  if (max_q_len > 0 && TT > max_q_len) TT = max_q_len;      // no sequence brings more rows than that
+  HE_REQUIRE(W <= SS_PRE * threads, "he_ssm_scan: a token's %d values do not fit a tile", W);
+  const size_t lds_bytes = (size_t)2 * TT * W * sizeof(float);
   const dim3 grid((P + PB - 1) / PB, R, num_seqs);
   hipStream_t s = (hipStream_t)stream;
-#define SCAN_LAUNCH(T, NPT)                                                                                   \
-  ssm_scan_kernel<T, NPT><<<grid, threads, 0, s>>>(                                                           \
+#define SCAN_LAUNCH(T, NPT)                                                                                       \
+  ssm_scan_kernel<T, NPT><<<grid, threads, lds_bytes, s>>>(                                                       \
       (float*)y_f32, (const T*)xbc, (const T*)dt_in, dt_stride, dt_bias, a_log, d_skip, w_dtype, (uint8_t*)state, \
-      state_stride, state_offset, (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, R, Q, N, P, NG, PB)
+      state_stride, state_offset, (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, R, Q, N, P, NG, PB, TT)
+  const int npt = ss_npt(N);
   if (dtype == HE_BF16) {
-    if (ss_npt(N) == 8) SCAN_LAUNCH(bf16_t, 8); else SCAN_LAUNCH(bf16_t, 16);
+    if (npt == 4) SCAN_LAUNCH(bf16_t, 4); else if (npt == 8) SCAN_LAUNCH(bf16_t, 8); else SCAN_LAUNCH(bf16_t, 16);
   } else {
-    if (ss_npt(N) == 8) SCAN_LAUNCH(float, 8); else SCAN_LAUNCH(float, 16);
+    if (npt == 4) SCAN_LAUNCH(float, 4); else if (npt == 8) SCAN_LAUNCH(float, 8); else SCAN_LAUNCH(float, 16);
   }
 #undef SCAN_LAUNCH
   return he_check_launch("he_ssm_scan");

@@ -586,11 +586,11 @@ def ssm_state_floats(R: int, P: int, N: int) -> int:
 
 @_op("ssm_scan")
 def ssm_scan(y, xbc, dt, dt_bias, a_log, d_skip, state, state_offset: int, cu_seqlens, seq_slot,
-             rows: int, num_seqs: int, R: int, Q: int, N: int, P: int) -> None:
+             rows: int, num_seqs: int, R: int, Q: int, N: int, P: int, max_q_len: int = 0) -> None:
     """y (fp32 [rows, R P]) = the selective scan of xbc [rows, R P + 2 Q N] (x, then B, then C) with step
     sizes softplus(dt + dt_bias) (dt: a view [rows, R] of wider rows), per head r the decay
     exp(-exp(a_log_r) dt) and the skip d_skip_r; the state [R][P][N'] lives at byte state_offset of a
-    sequence's row of `state` and is carried on."""
+    sequence's row of `state` and is carried on. max_q_len: a bound on the rows a sequence brings (0: none)."""
     C = R * P + 2 * Q * N
     _need(y, "y", torch.float32, (None, R * P))
     _need(xbc, "xbc", None, (None, C))
@@ -611,7 +611,7 @@ def ssm_scan(y, xbc, dt, dt_bias, a_log, d_skip, state, state_offset: int, cu_se
     _lib.check(L.he_ssm_scan(y.data_ptr(), xbc.data_ptr(), dt.data_ptr(), dt.stride(0), dt_bias.data_ptr(),
                              a_log.data_ptr(), d_skip.data_ptr(), dtype_code(dt_bias.dtype), state.data_ptr(),
                              state.stride(0), state_offset, cu_seqlens.data_ptr(), seq_slot.data_ptr(), rows,
-                             num_seqs, R, Q, N, P, dtype_code(xbc.dtype), _stream()))
+                             num_seqs, int(max_q_len), R, Q, N, P, dtype_code(xbc.dtype), _stream()))
 
 
 @_op("gated_group_norm")
@@ -634,22 +634,38 @@ def gated_group_norm(out, y, z, weight, rows: int, parts: int, eps: float) -> No
 
 @_op("route_tokens")
 def route_tokens(dense, ids, weights, logits, correction, rows: int, real: int, groups: int, keep: int,
-                 top: int, scale: float) -> None:
-    """The choice of `top` of E router outputs per row (logits fp32 [rows, E]): softmax scores s, the choice on
-    s + correction inside the `keep` best of `groups` equal groups, weights s * scale. dense (fp32
+                 top: int, scale: float, *, x=None, router=None) -> None:
+    """The choice of `top` of E router outputs per row (logits fp32 [rows, E]; or logits None and the kernel
+    forms them in fp32 from the rows x [rows, D] and the router's matrix, fp32 [E, D]): softmax scores s, the
+    choice on s + correction inside the `keep` best of `groups` equal groups, weights s * scale. dense (fp32
     [rows, real + 1]): each expert's weight or 0, the outputs from `real` on added up in the last column;
     ids (int32) and weights (fp32) [rows, top]: the chosen outputs."""
+    if logits is None:
+        E, D = router.shape
+        _need(router, "router", torch.float32)
+        _need(x, "x", None, (None, D))
+        if x.shape[0] < rows:
+            raise ValueError("route_tokens: x has fewer rows than the step")
+        return _route(dense, ids, weights, None, x, router, correction, rows, E, real, groups, keep, top, scale)
     E = logits.shape[-1]
     _need(logits, "logits", torch.float32, (None, E))
+    if logits.shape[0] < rows:
+        raise ValueError("route_tokens: buffers smaller than the row count")
+    _route(dense, ids, weights, logits, None, None, correction, rows, E, real, groups, keep, top, scale)
+
+
+def _route(dense, ids, weights, logits, x, router, correction, rows, E, real, groups, keep, top, scale) -> None:
     _need(dense, "dense", torch.float32, (None, real + 1))
     _need(ids, "ids", torch.int32, (None, top))
     _need(weights, "weights", torch.float32, (None, top))
     if correction is not None:
         _need(correction, "correction", None, (E,))
-    if min(logits.shape[0], dense.shape[0], ids.shape[0], weights.shape[0]) < rows:
+    if min(dense.shape[0], ids.shape[0], weights.shape[0]) < rows:
         raise ValueError("route_tokens: buffers smaller than the row count")
     L = _lib.load()
-    _lib.check(L.he_route_tokens(dense.data_ptr(), ids.data_ptr(), weights.data_ptr(), logits.data_ptr(),
+    _lib.check(L.he_route_tokens(dense.data_ptr(), ids.data_ptr(), weights.data_ptr(), _ptr(logits),
+                                 _ptr(x), dtype_code(x.dtype) if x is not None else F32, _ptr(router),
+                                 router.shape[1] if router is not None else 0,
                                  _ptr(correction), dtype_code(correction.dtype) if correction is not None else F32,
                                  rows, E, real, groups, keep, top, float(scale), _stream()))
 

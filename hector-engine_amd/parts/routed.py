@@ -11,8 +11,8 @@
     the I outputs without weights are identity experts: their result is n itself
     out = sum over the chosen outputs of weight * result
 
-How it runs: the router's product in fp32 (the weight is kept in 32-bit, the rows are widened), one
-kernel for the choice, and then the experts as one feed-forward: all gate and up rows side by side
+How it runs: one kernel for the router's product in fp32 (its matrix is kept in 32-bit) and the
+choice, and then the experts as one feed-forward: all gate and up rows side by side
 in one product, the activation kernel multiplies each expert's stretch by the token's weight for
 it (an exact 0 where it was not chosen) and appends weight * n for the identity experts, and one
 product with the down matrices side by side (and an identity block) adds everything up. Every step
@@ -63,7 +63,7 @@ class RoutedExperts(FeedForward):
         self._expert = names.get("expert", "experts.{e}.")
         self._sub = {k: names.get(k, d) for k, d in (("gate", "gate_proj.weight"), ("up", "up_proj.weight"),
                                                      ("down", "down_proj.weight"))}
-        self.router: Linear | None = None
+        self.router: torch.Tensor | None = None
         self.correction = None
         self.gate_up: Linear | None = None
         self.down: Linear | None = None
@@ -82,9 +82,8 @@ class RoutedExperts(FeedForward):
         return specs
 
     def bind(self, tensors):
-        # the router's sums are 32-bit whatever the run's precision: a weight kept in float32 runs
-        # through the plain product with the rows widened
-        self.router = Linear(tensors[self._router].to(torch.float32).contiguous())
+        # the router's sums are 32-bit whatever the run's precision: its matrix is kept in float32
+        self.router = tensors[self._router].to(torch.float32).contiguous()
         self.correction = tensors[self._correction] if self.has_correction else None
         gu, downs = [], []
         for e in range(self.real):
@@ -100,12 +99,12 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x, ctx: StepContext):
         rows, real, I = ctx.rows, self.real, self.inter
-        logits = self.router(x, rows, ctx, out_dtype=torch.float32)
         dense = ctx.alloc((rows, real + 1), torch.float32)
         ids = ctx.alloc((rows, self.top), torch.int32)
         weights = ctx.alloc((rows, self.top), torch.float32)
-        ops.route_tokens(dense, ids, weights, logits, self.correction, rows, real, self.groups, self.keep,
-                         self.top, self.scale)
+        # the router's product (fp32 sums over the rows as they are) and the choice, one launch
+        ops.route_tokens(dense, ids, weights, None, self.correction, rows, real, self.groups, self.keep,
+                         self.top, self.scale, x=x, router=self.router)
         cols = real * I + (self.hidden if self.identity else 0)
         act = {"alpha": self.alpha, "limit": self.limit, "up_shift": self.up_shift}
         if rows <= _ROW_CHUNK:

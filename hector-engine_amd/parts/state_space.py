@@ -69,14 +69,15 @@ class SelectiveScanMixer(Mixer):
         return self._conv_bytes() + 4 * self._scan_floats()
 
     def _scan_floats(self) -> int:
-        # the state dims are padded to the scan kernel's share per thread (8 dims up to 64, else 16,
-        # times a power of two of threads): the same rule as csrc/state_space.hip, kept here so that
-        # the cache can be sized where no kernel library is loaded
-        npt = 8 if self.N <= 64 else 16
+        # the state dims are padded to the scan kernel's share per thread (8 dims, 16 beyond 512, times a
+        # power of two of threads), the value dims to its workgroups' (256 threads at most): the same rule
+        # as csrc/state_space.hip, kept here so that the cache can be sized where no kernel library is loaded
+        npt = 8 if self.N <= 512 else 16
         ng = 1
         while ng * npt < self.N:
             ng *= 2
-        return self.R * self.P * ng * npt
+        pb = min(self.P, 256 // ng)
+        return self.R * -(-self.P // pb) * pb * ng * npt
 
     def tensor_specs(self):
         n = self._names
@@ -118,7 +119,7 @@ class SelectiveScanMixer(Mixer):
             y.zero_()           # the scan writes the rows of sequences only
         ops.ssm_scan(y, xbc, proj[:, inner + self.C:], self.dt_bias, self.a_log, self.d_skip, cache.state,
                      self._conv_bytes(), ctx.cu_seqlens, ctx.seq_slot, rows, ctx.num_seqs,
-                     self.R, self.Q, self.N, self.P)
+                     self.R, self.Q, self.N, self.P, max_q_len=ctx.max_q_len)
         g = ctx.alloc((rows, inner))
         ops.gated_group_norm(g, y, proj[:, :inner], self.norm, rows, self.parts, self.eps)
         return self.o_proj(g, rows, ctx, sink=ctx.take_sink())

@@ -103,7 +103,7 @@ def test_tensors_the_parts_ask_for_and_the_state_a_sequence_carries():
     plans = model.run_plans()
     # two carried inputs of 48 channels, then 3 x 8 x 16 floats of state (12 state dims in two shares of 8)
     assert plans[0].state_bytes == 0 and plans[1].state_bytes == 4 * (2 * 48 + 3 * 8 * 16)
-    # one carried input of 8 + 2 * 2 * 80 channels, then 2 x 4 x 128 floats (80 dims in eight shares of 16)
+    # one carried input of 8 + 2 * 2 * 80 channels, then 2 x 4 x 128 floats (80 dims in sixteen shares of 8)
     assert plans[2].state_bytes == 4 * 328 + 4 * 2 * 4 * 128
     # a differential attention keeps two keys a kv head, and the values once a map
     assert plans[0].kv.kv_heads == 4 and plans[1].kv is None
