@@ -134,7 +134,10 @@ static inline int ss_pb(int N, int P) {
   return P < most ? P : most;
 }
 
-template <typename T, int NPT>
+// TRIM: the tile is a small part of what the threads could stage (a one-token step), and the loops over a
+// thread's values end early. They are uniform branches, but behind branches the compiler waits for every load in
+// flight, so the long tiles of a prompt run without them.
+template <typename T, int NPT, bool TRIM>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(
     float* __restrict__ y, const T* __restrict__ xbc, const T* __restrict__ dt_in, int64_t dt_stride,
     const void* __restrict__ dt_bias, const void* __restrict__ a_log, const void* __restrict__ d_skip, int w_dtype,
@@ -172,59 +175,57 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
   const float dk = load_param(d_skip, r, w_dtype);
   const float db = load_param(dt_bias, r, w_dtype);
   const int tile_floats = TT * W;
-  // What thread `tid` stages of a tile does not change from tile to tile: value k is token tt_k's float j_k,
-  // which comes from column col_k of the token's row of xbc (B, C, x) or of dt_in (step size, decay), or is
-  // padding. The loads carry no branch (a padding value reads column 0 and is dropped), so that a tile's loads
-  // go out together and stay in flight while the tile before is computed; they are turned into values,
-  // softplus and decay included, when they are written to LDS.
-  enum { SS_ZERO = 0, SS_VALUE = 1, SS_DT = 2, SS_DECAY = 3 };
+  // What thread `tid` stages of a tile does not change from tile to tile: value k is token tok_of[k]'s float
+  // idx % W, which comes from column col[k] of the token's row of xbc (B, C, x), is padding (a zero), or is not
+  // this loop's (the two floats of a token's step size and decay: threads 0 .. 2 TT - 1 bring those). The loads
+  // carry no branch, so that a tile's loads go out together and stay in flight while the tile before is
+  // computed; they are turned into values when they are written to LDS.
+  enum { SS_SKIP = 0, SS_ZERO = 1, SS_VALUE = 2 };
   int col[SS_PRE], tok_of[SS_PRE];
   unsigned kinds = 0;                                  // two bits a value
 #pragma unroll
   for (int k = 0; k < SS_PRE; ++k) {
     col[k] = 0, tok_of[k] = 0;
-    if (k * threads >= tile_floats) break;             // (a one-token step stages a few hundred values, not thousands)
+    if (TRIM && k * threads >= tile_floats) break;
     const int idx = tid + k * threads;
     const int tt = idx / W, j = idx - tt * W;
-    int kind = SS_ZERO, c = 0;
-    if (idx < tile_floats) {
+    int kind = SS_SKIP, c = 0;
+    if (idx < tile_floats && j < 2 * Npad + PB) {
+      kind = SS_ZERO;
       if (j < Npad) {
         if (j < N) kind = SS_VALUE, c = inner + q * N + j;
       } else if (j < 2 * Npad) {
         if (j - Npad < N) kind = SS_VALUE, c = inner + (Q + q) * N + (j - Npad);
-      } else if (j < 2 * Npad + PB) {
-        if (p0 + (j - 2 * Npad) < P) kind = SS_VALUE, c = r * P + p0 + (j - 2 * Npad);
-      } else if (j < 2 * Npad + PB + 2) {
-        kind = j == 2 * Npad + PB ? SS_DT : SS_DECAY, c = r;
+      } else if (p0 + (j - 2 * Npad) < P) {
+        kind = SS_VALUE, c = r * P + p0 + (j - 2 * Npad);
       }
     }
     col[k] = c;
-    tok_of[k] = tt;
+    tok_of[k] = kind == SS_VALUE ? tt : 0;
     kinds |= (unsigned)kind << (2 * k);
   }
-  T pre[SS_PRE];
+  T pre[SS_PRE], pre_dt;
   auto fetch = [&](int first) {
+    const int last = t1 - 1 - first;                   // tokens beyond the sequence's rows read its last row
+    const T* base = xbc + (int64_t)first * C;
 #pragma unroll
     for (int k = 0; k < SS_PRE; ++k) {
-      if (k * threads >= tile_floats) break;           // (the same for the whole workgroup)
-      const int kind = (kinds >> (2 * k)) & 3;
-      const int t = min(first + tok_of[k], t1 - 1);
-      const T* src = kind >= SS_DT ? dt_in + (int64_t)t * dt_stride : xbc + (int64_t)t * C;
-      pre[k] = src[col[k]];
+      if (TRIM && k * threads >= tile_floats) break;
+      pre[k] = base[min(tok_of[k], last) * C + col[k]];
     }
+    pre_dt = dt_in[(int64_t)(first + min(min(tid >> 1, TT - 1), last)) * dt_stride + r];
   };
   auto put = [&](int buf) {
+    float* dst = lds + buf * tile_floats;
 #pragma unroll
     for (int k = 0; k < SS_PRE; ++k) {
-      if (k * threads >= tile_floats) break;
-      const int idx = tid + k * threads;
+      if (TRIM && k * threads >= tile_floats) break;
       const int kind = (kinds >> (2 * k)) & 3;
-      float v = kind == SS_ZERO ? 0.f : to_float(pre[k]);
-      if (kind >= SS_DT) {
-        const float dt = ss_softplus(v + db);
-        v = kind == SS_DT ? dt : expf(a * dt);
-      }
-      if (idx < tile_floats) lds[buf * tile_floats + idx] = v;
+      if (kind != SS_SKIP) dst[tid + k * threads] = kind == SS_ZERO ? 0.f : to_float(pre[k]);
+    }
+    if (tid < 2 * TT) {
+      const float dt = ss_softplus(to_float(pre_dt) + db);
+      dst[(tid >> 1) * W + 2 * Npad + PB + (tid & 1)] = (tid & 1) ? expf(a * dt) : dt;
     }
   };
   fetch(t0);
@@ -235,33 +236,57 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
     const bool more = first + TT < t1;
     if (more) fetch(first + TT);
     const int count = min(TT, t1 - first);
-    for (int tt = 0; tt < count; ++tt) {
-      const float* tok = lds + buf * tile_floats + tt * W;
-      const float x = tok[2 * Npad + pl];
-      const float dt = tok[2 * Npad + PB];
-      const float decay = tok[2 * Npad + PB + 1];
-      const float dtx = dt * x;
-      float acc = 0.f;
+    const float* mine = lds + buf * tile_floats + n0;                  // the thread's own B values of the tile's first token
+    const float* shared = lds + buf * tile_floats + 2 * Npad;          // x of the value dims, then dt and decay
+    float* ytile = y + (int64_t)first * inner + r * P + p0 + pl;
+    // two tokens a turn: their values are read from LDS together, their sums of y meet side by side. A turn
+    // whose second token lies beyond the rows runs it with decay 1 and step 0, which leaves S as it is.
+    for (int tt = 0; tt < count; tt += 2) {
+      const bool two = tt + 1 < count;
+      const int ta = tt * W, tb = (two ? tt + 1 : tt) * W;
+      float4 ba[NPT / 4], ca[NPT / 4], bb[NPT / 4], cb[NPT / 4];
 #pragma unroll
       for (int i4 = 0; i4 < NPT / 4; ++i4) {
-        const float4 b4 = *reinterpret_cast<const float4*>(tok + n0 + 4 * i4);
-        const float4 c4 = *reinterpret_cast<const float4*>(tok + Npad + n0 + 4 * i4);
-        const float b[4] = {b4.x, b4.y, b4.z, b4.w}, c[4] = {c4.x, c4.y, c4.z, c4.w};
+        ba[i4] = *reinterpret_cast<const float4*>(mine + ta + 4 * i4);
+        ca[i4] = *reinterpret_cast<const float4*>(mine + ta + Npad + 4 * i4);
+        bb[i4] = *reinterpret_cast<const float4*>(mine + tb + 4 * i4);
+        cb[i4] = *reinterpret_cast<const float4*>(mine + tb + Npad + 4 * i4);
+      }
+      const float xa = shared[ta + pl], xb = shared[tb + pl];
+      const float dta = shared[ta + PB], dtb = two ? shared[tb + PB] : 0.f;
+      const float da = shared[ta + PB + 1], dbb = two ? shared[tb + PB + 1] : 1.f;
+      const float dtxa = dta * xa, dtxb = dtb * xb;
+      float acca = 0.f, accb = 0.f;
+#pragma unroll
+      for (int i4 = 0; i4 < NPT / 4; ++i4) {
+        const float b[4] = {ba[i4].x, ba[i4].y, ba[i4].z, ba[i4].w}, c[4] = {ca[i4].x, ca[i4].y, ca[i4].z, ca[i4].w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          s[4 * i4 + e] = fmaf(decay, s[4 * i4 + e], dtx * b[e]);
-          acc = fmaf(s[4 * i4 + e], c[e], acc);
+          s[4 * i4 + e] = fmaf(da, s[4 * i4 + e], dtxa * b[e]);
+          acca = fmaf(s[4 * i4 + e], c[e], acca);
+        }
+      }
+#pragma unroll
+      for (int i4 = 0; i4 < NPT / 4; ++i4) {
+        const float b[4] = {bb[i4].x, bb[i4].y, bb[i4].z, bb[i4].w}, c[4] = {cb[i4].x, cb[i4].y, cb[i4].z, cb[i4].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s[4 * i4 + e] = fmaf(dbb, s[4 * i4 + e], dtxb * b[e]);
+          accb = fmaf(s[4 * i4 + e], c[e], accb);
         }
       }
       // the NG neighbouring lanes of a value dim: through the vector ALU's own lane exchanges (every lane
       // of the wavefront runs this loop, which they require)
-      if (NG > 1) acc += lane_xor1(acc);
-      if (NG > 2) acc += lane_xor2(acc);
-      if (NG > 4) acc += lane_xor4(acc);
-      if (NG > 8) acc += lane_xor8(acc);
-      if (NG > 16) acc = xor16_sum(acc);
-      if (NG > 32) acc = xor32_sum(acc);
-      if (ng == 0 && live) y[(int64_t)(first + tt) * inner + r * P + p0 + pl] = fmaf(dk, x, acc);
+      if (NG > 1) acca += lane_xor1(acca), accb += lane_xor1(accb);
+      if (NG > 2) acca += lane_xor2(acca), accb += lane_xor2(accb);
+      if (NG > 4) acca += lane_xor4(acca), accb += lane_xor4(accb);
+      if (NG > 8) acca += lane_xor8(acca), accb += lane_xor8(accb);
+      if (NG > 16) acca = xor16_sum(acca), accb = xor16_sum(accb);
+      if (NG > 32) acca = xor32_sum(acca), accb = xor32_sum(accb);
+      if (ng == 0 && live) {
+        ytile[(int64_t)tt * inner] = fmaf(dk, xa, acca);
+        if (two) ytile[(int64_t)(tt + 1) * inner] = fmaf(dk, xb, accb);
+      }
     }
     if (more) put(buf ^ 1);
     __syncthreads();
@@ -300,20 +325,25 @@ extern "C" int he_ssm_scan(void* y_f32, const void* xbc, const void* dt_in, int6
   TT = TT < 1 ? 1 : (TT > 16 ? 16 : TT);
   if (max_q_len > 0 && TT > max_q_len) TT = max_q_len;      // no sequence brings more rows than that
   HE_REQUIRE(W <= SS_PRE * threads, "he_ssm_scan: a token's %d values do not fit a tile", W);
+  if (2 * TT > threads) TT = threads / 2;               // a thread a token brings its step size, another its decay
   const size_t lds_bytes = (size_t)2 * TT * W * sizeof(float);
   const dim3 grid((P + PB - 1) / PB, R, num_seqs);
   hipStream_t s = (hipStream_t)stream;
+  const bool trim = TT * W <= (SS_PRE / 2) * threads;
 #define SCAN_LAUNCH(T, NPT)                                                                                       \
-  ssm_scan_kernel<T, NPT><<<grid, threads, lds_bytes, s>>>(                                                       \
+  if (trim) SCAN_LAUNCH_(T, NPT, true); else SCAN_LAUNCH_(T, NPT, false)
+#define SCAN_LAUNCH_(T, NPT, TRIM)                                                                                \
+  ssm_scan_kernel<T, NPT, TRIM><<<grid, threads, lds_bytes, s>>>(                                                       \
       (float*)y_f32, (const T*)xbc, (const T*)dt_in, dt_stride, dt_bias, a_log, d_skip, w_dtype, (uint8_t*)state, \
       state_stride, state_offset, (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, R, Q, N, P, NG, PB, TT)
   const int npt = ss_npt(N);
   if (dtype == HE_BF16) {
-    if (npt == 4) SCAN_LAUNCH(bf16_t, 4); else if (npt == 8) SCAN_LAUNCH(bf16_t, 8); else SCAN_LAUNCH(bf16_t, 16);
+    if (npt == 8) { SCAN_LAUNCH(bf16_t, 8); } else { SCAN_LAUNCH(bf16_t, 16); }
   } else {
-    if (npt == 4) SCAN_LAUNCH(float, 4); else if (npt == 8) SCAN_LAUNCH(float, 8); else SCAN_LAUNCH(float, 16);
+    if (npt == 8) { SCAN_LAUNCH(float, 8); } else { SCAN_LAUNCH(float, 16); }
   }
 #undef SCAN_LAUNCH
+#undef SCAN_LAUNCH_
   return he_check_launch("he_ssm_scan");
 }
 
