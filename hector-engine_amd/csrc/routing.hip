@@ -219,6 +219,40 @@ __global__ void routed_act_kernel(T* __restrict__ out, const T* __restrict__ gat
   out[row * (int64_t)cols + j] = from_float<T>(v);
 }
 
+// The same for bf16 rows, eight columns a thread (16-byte loads and stores): needs I and extra in multiples of 8.
+template <bool CLAMPED>
+__global__ void routed_act_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ gate_up,
+                                      const float* __restrict__ dense, const uint16_t* __restrict__ h, int real, int I,
+                                      int extra, GatedAct act) {
+  const int64_t row = blockIdx.y;
+  const int cols = real * I + extra;
+  const int j = 8 * (blockIdx.x * blockDim.x + threadIdx.x);
+  if (j >= cols) return;
+  const float* d = dense + row * (real + 1);
+  float v[8];
+  if (j < real * I) {
+    const float w = d[j / I];
+    const uint4* gu = reinterpret_cast<const uint4*>(gate_up + row * (int64_t)(2 * real * I) + 2 * j);
+    const uint4 lo = gu[0], hi = gu[1];
+    const uint32_t pairs[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};      // (gate, up) a word
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      v[i] = w == 0.f ? 0.f
+                      : he_gated_act<CLAMPED>(__uint_as_float(pairs[i] << 16), __uint_as_float(pairs[i] & 0xffff0000u), act) * w;
+  } else {
+    const float w = d[real];
+    const uint4 raw = *reinterpret_cast<const uint4*>(h + row * (int64_t)extra + (j - real * I));
+    const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = w == 0.f ? 0.f : w * __uint_as_float(words[i] << 16);
+      v[2 * i + 1] = w == 0.f ? 0.f : w * __uint_as_float(words[i] & 0xffff0000u);
+    }
+  }
+  *reinterpret_cast<uint4*>(out + row * (int64_t)cols + j) =
+      make_uint4(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7]));
+}
+
 extern "C" int he_routed_act(void* out, const void* gate_up, const void* dense_f32, const void* h, int rows, int real,
                              int I, int extra, int dtype, float alpha, float limit, float up_shift, void* stream) {
   HE_REQUIRE(rows >= 0 && real >= 0 && I > 0 && extra >= 0 && (int64_t)real * I + extra > 0, "he_routed_act: bad sizes");
@@ -230,6 +264,17 @@ extern "C" int he_routed_act(void* out, const void* gate_up, const void* dense_f
   hipStream_t s = (hipStream_t)stream;
   const bool clamped = limit > 0.f || alpha != 1.f || up_shift != 0.f;
   const GatedAct act = {alpha, limit > 0.f ? limit : INFINITY, up_shift};
+  if (dtype == HE_BF16 && I % 8 == 0 && extra % 8 == 0 &&
+      ((((uintptr_t)out) | ((uintptr_t)gate_up) | ((uintptr_t)h)) & 15) == 0) {
+    const dim3 vgrid((cols / 8 + 255) / 256, rows);
+    if (clamped)
+      routed_act_vec_kernel<true><<<vgrid, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)gate_up, (const float*)dense_f32,
+                                                        (const uint16_t*)h, real, I, extra, act);
+    else
+      routed_act_vec_kernel<false><<<vgrid, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)gate_up, (const float*)dense_f32,
+                                                         (const uint16_t*)h, real, I, extra, act);
+    return he_check_launch("he_routed_act");
+  }
 #define ACT_LAUNCH(T, CL)                                                                                      \
   routed_act_kernel<T, CL><<<grid, 256, 0, s>>>((T*)out, (const T*)gate_up, (const float*)dense_f32, (const T*)h, real, \
                                                 I, extra, act)

@@ -304,6 +304,10 @@ MODELS = {
            "layers": [layer("attention", attn(6, 1, 8, 40, 0.35, 0.3, (1.0, 1)), moe(9, 3, 4, 32, 1.0, 3, 1, 1.5)),
                       layer("attention", attn(2, 2, 32, 32, 0.18, 0.6, (0.5, 70)), moe(2, 0, 2, 56, 1.0)),
                       layer("mamba2", scan(5, 8, 64, 1, 1, 5), moe(3, 1, 1, 24, 2.0, 2, 1, 1.0))]},
+    # no attention at all (a cache without keys and values), value dims that fill more than one workgroup
+    "P4": {"architecture": "Penasun", "vocab": 75, "width": 32, "norm": {"eps": 1e-6},
+           "layers": [layer("mamba2", scan(2, 72, 32, 2, 4, 2), moe(2, 2, 2, 16, 1.0, 2, 2, 1.0)),
+                      layer("mamba2", scan(4, 4, 8, 1, 2, 1))]},
 }
 
 
