@@ -64,12 +64,15 @@ def run_schedule(slots, per_step):
 
 # ------------------------------------------------------------------ convolution with carried inputs
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C,K", [(10, 1), (37, 2), (300, 4), (64, 7)])
-def test_convolution_in_portions_and_batches_equals_the_whole(ops, dtype, C, K):
+@pytest.mark.parametrize("C,K,col0", [(10, 1, 2), (37, 2, 2), (300, 4, 2), (64, 7, 2), (64, 4, 8), (2112, 3, 8), (72, 1, 0)])
+def test_convolution_in_portions_and_batches_equals_the_whole(ops, dtype, C, K, col0):
+    """col0: the column the channels begin at in their rows (also 8 and 0, in rows of a multiple of 8 columns:
+    aligned rows as a model of usual sizes has them)."""
     dt = TORCH[dtype]
-    u = [rnd(n, C + 5, seed=3 + i).to(dt) for i, n in enumerate(LENGTHS)]       # rows wider than the channels read
+    wide = C + (5 if col0 == 2 else 16)
+    u = [rnd(n, wide, seed=3 + i).to(dt) for i, n in enumerate(LENGTHS)]       # rows wider than the channels read
     taps, bias = rnd(C, K, seed=1, scale=0.5).to(dt), rnd(C, seed=2).to(dt)
-    want = [P.causal_conv(x[:, 2:2 + C].double(), taps.double(), bias.double())[0] for x in u]
+    want = [P.causal_conv(x[:, col0:col0 + C].double(), taps.double(), bias.double())[0] for x in u]
     slots = [4, 0, 2]                                                          # not in order, with gaps
     state = torch.zeros(6, 4 * (K - 1) * C + 64, dtype=torch.uint8, device="cuda")
     state[:, 4 * (K - 1) * C:] = 77                                            # what lies behind is not touched
@@ -79,7 +82,7 @@ def test_convolution_in_portions_and_batches_equals_the_whole(ops, dtype, C, K):
         x = torch.cat([u[s][at:at + n] for s, n, at in zip(seqs, q_lens, starts)])
         rows = x.shape[0]
         out = torch.empty(rows, C, dtype=dt, device="cuda")
-        ops.conv_state(out, dev(x)[:, 2:2 + C], dev(taps), dev(bias), state, *step_meta(q_lens, starts, sl),
+        ops.conv_state(out, dev(x)[:, col0:col0 + C], dev(taps), dev(bias), state, *step_meta(q_lens, starts, sl),
                        rows, len(seqs), all(n == 1 for n in q_lens))
         at = 0
         for s, n, st in zip(seqs, q_lens, starts):
