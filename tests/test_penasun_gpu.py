@@ -311,6 +311,10 @@ MODELS = {
     "P4": {"architecture": "Penasun", "vocab": 75, "width": 32, "norm": {"eps": 1e-6},
            "layers": [layer("mamba2", scan(2, 72, 32, 2, 4, 2), moe(2, 2, 2, 16, 1.0, 2, 2, 1.0)),
                       layer("mamba2", scan(4, 4, 8, 1, 2, 1))]},
+    # sizes that are no multiple of 8 anywhere: under bfloat16 every product takes the plain kernel
+    "P5": {"architecture": "Penasun", "vocab": 50, "width": 36, "norm": {"eps": 1e-5},
+           "layers": [layer("mamba2", scan(3, 12, 10, 3, 3, 2), moe(3, 1, 2, 10, 1.0, 2, 1, 1.2)),
+                      layer("attention", attn(2, 1, 12, 20, 0.3, 0.45, (0.7, 5)), moe(3, 1, 2, 10, 1.0, 2, 1, 1.2))]},
 }
 
 
