@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 24
+#define HE_ABI_VERSION 25
 
 #ifdef __cplusplus
 extern "C" {
@@ -238,6 +238,15 @@ int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32, const voi
                     int top, float scale, void* stream);
 int he_routed_act(void* out, const void* gate_up, const void* dense_f32, const void* h, int rows, int real,
                   int I, int extra, int dtype, float alpha, float limit, float up_shift, void* stream);
+// For a step of very few rows (bf16): out[rows][D] = the weighted sum of the chosen experts' results alone, from
+// the same fused matrices the products over all experts use (gate_up [2 real I][D], rows alternating gate and up;
+// down [D][ldw] with the experts' matrices side by side), plus dense[row][real] * x (the identity experts' share).
+// ids / weights [rows][top] and dense [rows][real + 1] as he_route_tokens leaves them; h_scratch: rows * top * I
+// elements. I, D and ldw in multiples of 8.
+int he_chosen_experts(void* out, void* h_scratch, const void* x, const void* gate_up, const void* down,
+                      int64_t ldw, const void* ids_i32, const void* weights_f32, const void* dense_f32,
+                      int rows, int top, int real, int I, int D, float alpha, float limit, float up_shift,
+                      void* stream);
 int he_diff_heads(void* out, const void* attn, int rows, int H, int G, int hd, int vd, float lambda,
                   float post, float eps, int dtype, void* stream);
 

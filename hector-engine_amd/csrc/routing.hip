@@ -287,6 +287,110 @@ extern "C" int he_routed_act(void* out, const void* gate_up, const void* dense_f
   return he_check_launch("he_routed_act");
 }
 
+// ---- the chosen experts alone, for steps of very few rows ---------------------------------------
+// Where a step's rows choose fewer experts than there are, the two products over all experts read weights
+// nobody asked for. These two kernels walk only the chosen experts' rows of the same fused matrices (bf16):
+// a wavefront an output, the lanes along K with 16-byte loads, sums in fp32.
+__device__ __forceinline__ float dot8_bf16(const uint4& a, const uint4& b, float acc) {
+  const uint32_t x[4] = {a.x, a.y, a.z, a.w}, y[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    acc = fmaf(__uint_as_float(x[i] << 16), __uint_as_float(y[i] << 16), acc);
+    acc = fmaf(__uint_as_float(x[i] & 0xffff0000u), __uint_as_float(y[i] & 0xffff0000u), acc);
+  }
+  return acc;
+}
+
+// h[(row, k), i] = weight[row, k] * act(gate . x[row], up . x[row]) with gate and up the rows 2 (e I + i) and
+// 2 (e I + i) + 1 of gate_up [2 real I][D], e = ids[row, k]; zeros where e is no expert with weights.
+template <bool CLAMPED>
+__global__ __launch_bounds__(256) void chosen_gate_up_kernel(uint16_t* __restrict__ h, const uint16_t* __restrict__ x,
+                                                             const uint16_t* __restrict__ gate_up,
+                                                             const int32_t* __restrict__ ids,
+                                                             const float* __restrict__ weights, int top, int real, int I,
+                                                             int D, GatedAct act) {
+  const int lane = threadIdx.x & 63;
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t rk = blockIdx.y;                 // row * top + k
+  if (i >= I) return;
+  const int e = ids[rk];
+  const int64_t row = rk / top;
+  float g = 0.f, u = 0.f;
+  if (e >= 0 && e < real) {
+    const uint16_t* wg = gate_up + ((int64_t)e * I + i) * 2 * D;
+    const uint16_t* xr = x + row * D;
+#pragma unroll 4
+    for (int c = lane * 8; c < D; c += 512) {
+      const uint4 xv = *reinterpret_cast<const uint4*>(xr + c);
+      g = dot8_bf16(*reinterpret_cast<const uint4*>(wg + c), xv, g);
+      u = dot8_bf16(*reinterpret_cast<const uint4*>(wg + D + c), xv, u);
+    }
+  }
+  g = wave_sum(g);
+  u = wave_sum(u);
+  if (lane == 0) {
+    const float v = (e >= 0 && e < real) ? he_gated_act<CLAMPED>(g, u, act) * weights[rk] : 0.f;
+    h[rk * I + i] = float_to_bf16_bits(v);
+  }
+}
+
+// out[row, d] = sum over the row's chosen experts e of down[d][e I ..] . h[(row, k)] + dense[row][real] * x[row, d]
+// (down [D][ldw]: the experts' matrices side by side; the last term is the identity experts' share).
+__global__ __launch_bounds__(256) void chosen_down_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ h,
+                                                          const uint16_t* __restrict__ x, const uint16_t* __restrict__ down,
+                                                          int64_t ldw, const int32_t* __restrict__ ids,
+                                                          const float* __restrict__ dense, int top, int real, int I,
+                                                          int D) {
+  const int lane = threadIdx.x & 63;
+  const int d = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t row = blockIdx.y;
+  if (d >= D) return;
+  float acc = 0.f;
+  for (int k = 0; k < top; ++k) {
+    const int e = ids[row * top + k];
+    if (e < 0 || e >= real) continue;
+    const uint16_t* w = down + (int64_t)d * ldw + (int64_t)e * I;
+    const uint16_t* hr = h + (row * top + k) * I;
+#pragma unroll 4
+    for (int c = lane * 8; c < I; c += 512)
+      acc = dot8_bf16(*reinterpret_cast<const uint4*>(w + c), *reinterpret_cast<const uint4*>(hr + c), acc);
+  }
+  acc = wave_sum(acc);
+  if (lane == 0)
+    out[row * D + d] = float_to_bf16_bits(fmaf(dense[row * (real + 1) + real], bf16_bits_to_float(x[row * D + d]), acc));
+}
+
+extern "C" int he_chosen_experts(void* out, void* h_scratch, const void* x, const void* gate_up, const void* down,
+                                 int64_t ldw, const void* ids_i32, const void* weights_f32, const void* dense_f32,
+                                 int rows, int top, int real, int I, int D, float alpha, float limit, float up_shift,
+                                 void* stream) {
+  HE_REQUIRE(rows >= 0 && top > 0 && real > 0 && I > 0 && D > 0, "he_chosen_experts: bad sizes");
+  HE_REQUIRE(I % 8 == 0 && D % 8 == 0 && ldw % 8 == 0 && ldw >= (int64_t)real * I,
+             "he_chosen_experts: I=%d, D=%d and the down matrix's row stride must be multiples of 8", I, D);
+  HE_REQUIRE(((((uintptr_t)out) | ((uintptr_t)h_scratch) | ((uintptr_t)x) | ((uintptr_t)gate_up) | ((uintptr_t)down)) & 15) == 0,
+             "he_chosen_experts: pointers must be 16-byte aligned");
+  HE_REQUIRE((int64_t)rows * top <= 65535, "he_chosen_experts: too many rows");
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const bool clamped = limit > 0.f || alpha != 1.f || up_shift != 0.f;
+  const GatedAct act = {alpha, limit > 0.f ? limit : INFINITY, up_shift};
+  const dim3 grid_up((I + 3) / 4, rows * top);
+  if (clamped)
+    chosen_gate_up_kernel<true><<<grid_up, 256, 0, s>>>((uint16_t*)h_scratch, (const uint16_t*)x, (const uint16_t*)gate_up,
+                                                        (const int32_t*)ids_i32, (const float*)weights_f32, top, real, I,
+                                                        D, act);
+  else
+    chosen_gate_up_kernel<false><<<grid_up, 256, 0, s>>>((uint16_t*)h_scratch, (const uint16_t*)x, (const uint16_t*)gate_up,
+                                                         (const int32_t*)ids_i32, (const float*)weights_f32, top, real, I,
+                                                         D, act);
+  int st = he_check_launch("he_chosen_experts (gate, up)");
+  if (st) return st;
+  chosen_down_kernel<<<dim3((D + 3) / 4, rows), 256, 0, s>>>((uint16_t*)out, (const uint16_t*)h_scratch, (const uint16_t*)x,
+                                                             (const uint16_t*)down, ldw, (const int32_t*)ids_i32,
+                                                             (const float*)dense_f32, top, real, I, D);
+  return he_check_launch("he_chosen_experts (down)");
+}
+
 // Differential attention's last step. attn [rows][2 H][hd] holds, for kv head g and its R = H / G
 // query heads, first the R outputs of score map 1 and then the R outputs of map 2 (head order
 // [g][map][r]); out [rows][H][vd], head h = g R + r:

@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 24
+EXPECTED_ABI = 25
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -65,6 +65,8 @@ _SIGNATURES = {
     "he_route_tokens": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_int, c_ptr, c_int, c_int, c_int, c_int,
                         c_int, c_int, c_int, c_f32, c_ptr],
     "he_routed_act": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_f32, c_ptr],
+    "he_chosen_experts": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int,
+                          c_int, c_f32, c_f32, c_f32, c_ptr],
     "he_diff_heads": [c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_f32, c_int, c_ptr],
     "he_attention_plain_workspace_floats": [c_int, c_int, c_int, c_int, c_int, c_int],
     "he_attention_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int,

@@ -689,6 +689,31 @@ def routed_act(out, gate_up, dense, h, rows: int, real: int, inter: int, *, alph
                                extra, dtype_code(out.dtype), float(alpha), float(limit), float(up_shift), _stream()))
 
 
+@_op("chosen_experts")
+def chosen_experts(out, h_scratch, x, gate_up, down, ids, weights, dense, rows: int, real: int, inter: int, *,
+                   alpha: float = 1.0, limit: float = 0.0, up_shift: float = 0.0) -> None:
+    """For a step of very few bf16 rows: out[rows, D] = the weighted sum of the chosen experts' results alone
+    (ids, weights [rows, top] and dense [rows, real + 1] as route_tokens leaves them), read from the fused matrices
+    of the products over all experts: gate_up [2 real inter, D] (gate and up alternating), down [D, real inter (+ D)].
+    The identity experts' share dense[row, real] * x is added. h_scratch: bf16 [rows * top, inter]."""
+    D = x.shape[1]
+    top = ids.shape[1]
+    for name, t in (("out", out), ("h_scratch", h_scratch), ("x", x), ("gate_up", gate_up), ("down", down)):
+        _need(t, name, torch.bfloat16)
+    _need(ids, "ids", torch.int32, (None, top))
+    _need(weights, "weights", torch.float32, (None, top))
+    _need(dense, "dense", torch.float32, (None, real + 1))
+    if tuple(gate_up.shape) != (2 * real * inter, D) or down.shape[0] != D or down.shape[1] < real * inter:
+        raise ValueError("chosen_experts: the fused matrices do not match the sizes")
+    if min(out.shape[0], x.shape[0], ids.shape[0], weights.shape[0], dense.shape[0]) < rows or out.shape[1] != D \
+            or h_scratch.numel() < rows * top * inter:
+        raise ValueError("chosen_experts: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_chosen_experts(out.data_ptr(), h_scratch.data_ptr(), x.data_ptr(), gate_up.data_ptr(), down.data_ptr(),
+                                   down.stride(0), ids.data_ptr(), weights.data_ptr(), dense.data_ptr(), rows, top, real,
+                                   inter, D, float(alpha), float(limit), float(up_shift), _stream()))
+
+
 @_op("diff_heads")
 def diff_heads(out, attn, rows: int, H: int, G: int, hd: int, vd: int, lam: float, post: float, eps: float) -> None:
     """out[rows, H, vd] = rms(a1 - lam * a2) * post per head, a1 and a2 the outputs of the two score maps in

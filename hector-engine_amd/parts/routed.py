@@ -17,7 +17,8 @@ in one product, the activation kernel multiplies each expert's stretch by the to
 it (an exact 0 where it was not chosen) and appends weight * n for the identity experts, and one
 product with the down matrices side by side (and an identity block) adds everything up. Every step
 has the same launches whatever the tokens choose, so it replays as a graph, and a token's sums do
-not depend on the rest of the batch.
+not depend on the rest of the batch. A bfloat16 step of so few rows that they cannot choose more than
+half of the experts reads only the chosen experts' rows of the same matrices (ops.chosen_experts).
 names: the suffixes of its tensors (router, correction; expert e's are 'e<e>.' + gate / up / down).
 """
 from __future__ import annotations
@@ -97,6 +98,13 @@ class RoutedExperts(FeedForward):
         self.gate_up = Linear(torch.cat(gu, 0).contiguous())
         self.down = Linear(torch.cat(downs, 1).contiguous())
 
+    def _few_rows(self, rows: int, x, ctx: StepContext) -> bool:
+        """Whether the step runs through the chosen experts alone (kernels.ops.chosen_experts): bfloat16 with the
+        fast kernels, sizes in multiples of 8, and so few rows that they cannot choose more than half of the
+        experts. (The 32-bit path keeps the products over all experts, whose sums do not depend on the batch.)"""
+        return (ctx.env.fast_kernels and x.dtype == torch.bfloat16 and self.gate_up.weight.dtype == torch.bfloat16
+                and self.inter % 8 == 0 and self.hidden % 8 == 0 and 2 * rows * self.top <= self.real)
+
     def forward(self, x, ctx: StepContext):
         rows, real, I = ctx.rows, self.real, self.inter
         dense = ctx.alloc((rows, real + 1), torch.float32)
@@ -107,6 +115,12 @@ class RoutedExperts(FeedForward):
                          self.top, self.scale, x=x, router=self.router)
         cols = real * I + (self.hidden if self.identity else 0)
         act = {"alpha": self.alpha, "limit": self.limit, "up_shift": self.up_shift}
+        if self._few_rows(rows, x, ctx):
+            # the rows of the step choose at most half of the experts: only those experts' weights are read
+            h = ctx.alloc((rows * self.top, I))
+            out = ctx.alloc((rows, self.hidden))
+            ops.chosen_experts(out, h, x, self.gate_up.weight, self.down.weight, ids, weights, dense, rows, real, I, **act)
+            return out
         if rows <= _ROW_CHUNK:
             gu = self.gate_up(x, rows, ctx)
             h = ctx.alloc((rows, cols))

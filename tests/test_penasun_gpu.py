@@ -246,6 +246,39 @@ def test_weighted_expert_activation(ops, dtype, rows, real, I, extra):
     assert torch.allclose(out.cpu().double(), want, rtol=tol, atol=tol)
 
 
+@pytest.mark.parametrize("rows,real,identity,top,I,D", [(2, 5, 1, 2, 24, 40), (1, 16, 2, 4, 64, 128), (3, 12, 0, 2, 8, 16)])
+def test_the_chosen_experts_alone_give_the_weighted_sum(ops, rows, real, identity, top, I, D):
+    """The path of steps of very few rows, which reads only the chosen experts' weights, against the plain experts."""
+    E = real + identity
+    bf = torch.bfloat16
+    x = rnd(rows, D, seed=1).to(bf)
+    gates = [rnd(I, D, seed=10 + e, scale=0.3).to(bf) for e in range(real)]
+    ups = [rnd(I, D, seed=40 + e, scale=0.3).to(bf) for e in range(real)]
+    downs = [rnd(D, I, seed=70 + e, scale=0.3).to(bf) for e in range(real)]
+    router = rnd(E, D, seed=5, scale=0.5)
+    if identity:
+        router[real] = 4 * x[0].float()              # row 0 chooses an identity expert for certain
+    gate_up = torch.cat([torch.stack([g, u], 1).reshape(2 * I, D) for g, u in zip(gates, ups)], 0).contiguous()
+    down = torch.cat(downs + ([torch.eye(D, dtype=bf)] if identity else []), 1).contiguous()
+    dense = torch.empty(rows, real + 1, device="cuda")
+    ids = torch.empty(rows, top, dtype=torch.int32, device="cuda")
+    weights = torch.empty(rows, top, device="cuda")
+    ops.route_tokens(dense, ids, weights, None, None, rows, real, 1, 1, top, 1.5, x=dev(x), router=dev(router))
+    out = torch.empty(rows, D, dtype=bf, device="cuda")
+    h = torch.empty(rows * top, I, dtype=bf, device="cuda")
+    ops.chosen_experts(out, h, dev(x), dev(gate_up), dev(down), ids, weights, dense, rows, real, I,
+                       alpha=1.702, limit=1.0, up_shift=1.0)
+    want = torch.zeros(rows, D, dtype=torch.float64)
+    for r in range(rows):
+        for e, w in zip(ids[r].tolist(), weights[r].tolist()):
+            if e >= real:
+                want[r] += w * x[r].double()
+            else:
+                want[r] += w * P.bounded_expert(x[r].double(), gates[e].double(), ups[e].double(), downs[e].double(), 1.0)
+    assert identity == 0 or real in ids[0].tolist()
+    assert torch.allclose(out.cpu().double(), want, rtol=2 ** -6, atol=2 ** -6 * want.abs().max().item())
+
+
 # ------------------------------------------------------------------ differential heads, query temperature
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,hd,vd", [(4, 2, 64, 64), (6, 1, 48, 40), (3, 3, 16, 8), (2, 2, 128, 100)])
