@@ -21,10 +21,10 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 // logits[e] = sum_i x[row][i] * router[e][i] in fp32 (router fp32 [E][D]; a lane adds its elements i = lane,
 // lane + 64, ... in that order, the lanes' sums meet in the wavefront's butterfly: one fixed order a row,
 // whatever else the step holds). s = softmax(logits) over all E outputs; the choice is made
-// on c = s + correction: the E outputs form `groups` equal groups of neighbours, a group counts by its
-// largest c, only the outputs of the `keep` best groups can be chosen (the others count as -inf), and
-// the `top` largest c among those are chosen. The weight of a chosen output is s * scale (not c, and
-// not renormalised). The last E - real outputs are experts without weights whose result is the input
+// on c = s + correction: the E outputs are cut into `groups` equal runs of neighbours, each run ranked by the
+// largest c it holds; outside the `keep` best runs every c is replaced by -inf, and the `top` largest c that
+// are left are chosen. The weight of a chosen output is s * scale (s, not c; the weights are not made to sum
+// to one). The last E - real outputs are experts without weights whose result is the input
 // itself: their weights are added up in column `real` of dense. dense [rows][real + 1] holds the
 // weight of every expert (0 where not chosen); ids / weights [rows][top] list the chosen ones.
 #define ROUTE_WAVES 8

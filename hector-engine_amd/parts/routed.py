@@ -3,9 +3,9 @@
     z = W_router n                    fp32, E + I outputs: E experts with weights, then I without
     s = softmax(z)                    over all outputs
     c = s + correction                the choice is made on c, the weights on s
-    the outputs form `groups` equal groups of neighbours; a group counts by its largest c, and only
-    outputs of the `keep` best groups can be chosen (the others count as -inf); the `top` largest c
-    among them are chosen, and a chosen output weighs s * scale (not renormalised)
+    the outputs are cut into `groups` equal runs of neighbours, each run ranked by the largest c it
+    holds; outside the `keep` best runs every c is replaced by -inf; the `top` largest c that are left
+    are chosen, and a chosen output weighs s * scale (the weights are not made to sum to one)
     expert e: g = min(W_gate n, limit), u = clamp(W_up n, -limit, limit),
               y = g * sigmoid(alpha g) * (u + 1), result W_down y          (no biases)
     the I outputs without weights are identity experts: their result is n itself
