@@ -349,8 +349,8 @@ extern "C" int he_ssm_scan(void* y_f32, const void* xbc, const void* dt_in, int6
 
 // ---- gated, grouped RMS norm ------------------------------------------------------------------
 // out[row, c] = v / sqrt(mean over c's part of v^2 + eps) * weight[c], v = y[row, c] * silu(z[row, c]):
-// the gate comes before the norm, and each of the `parts` equal stretches of a row has a root mean
-// square of its own. One workgroup a (row, part).
+// the product with silu(z) is formed first and normalised afterwards, each of the `parts` equal stretches of
+// a row by a root mean square of its own. One workgroup a (row, part).
 template <typename T>
 __global__ void gated_group_norm_kernel(T* __restrict__ out, const float* __restrict__ y, const T* __restrict__ z,
                                         int64_t z_stride, const void* __restrict__ weight, int w_dtype, int W,

@@ -22,9 +22,9 @@ Options of the same part, each off unless its parameter says otherwise:
   head_gate   head h's output is multiplied by sigmoid(g_h), g = Wg n with one row of Wg a head;
               the rows of Wg ride behind q||k||v in the one product.
   q_temp      {coef, every}: the q of position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).
-  score_maps  2: differential attention. A head has two queries and a kv head two keys (the rows of
-              the q and k matrices lie head by head as [map 1, map 2]); each map is a softmax attention
-              of its own over the same values, a1 and a2, and the head's output is
+  score_maps  2: differential attention. A head has two queries and a kv head two keys (in the q and k
+              matrices a head's rows for map 1 stand in front of its rows for map 2); the two maps are
+              separate softmax attentions that share the head's values, with results a1 and a2, and the head's output is
               rms(a1 - lambda * a2) * (1 - diff) over its value_dim values (no gain, eps `diff_eps`), with
               lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff from four stored vectors of head_dim and the
               constant `diff`. The kernels see 2 H heads over 2 KVH kv heads: the rows of q are reordered
